@@ -1,5 +1,6 @@
-"""Typed configurations and the architecture registry; importing registers "llama"."""
+"""Typed configurations and the architecture registry; importing registers "llama" and "Sunusun"."""
 from .base import (Architecture, ConfigError, architecture_for, architecture_names, load_config,
                    read_config_json, register_architecture)
 from .llama import LlamaConfig, RopeScaling
+from .sunusun import SunusunConfig
 from . import llama_plan  # noqa: F401  (registration)

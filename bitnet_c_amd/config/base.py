@@ -44,11 +44,13 @@ def architecture_names():
 
 
 def architecture_for(raw: dict) -> Architecture:
-    """Choose by `model_type`, then by the entries of `architectures`."""
+    """Choose by `model_type`, then by the entries of `architectures`, then by `architecture`."""
     keys = []
     if raw.get("model_type"):
         keys.append(str(raw["model_type"]))
     keys += [str(a) for a in raw.get("architectures") or []]
+    if isinstance(raw.get("architecture"), str):
+        keys.append(raw["architecture"])
     for key in keys:
         if key in _ARCHITECTURES:
             return _ARCHITECTURES[key]
@@ -69,10 +71,29 @@ def read_config_json(folder: str) -> dict:
 
 
 def load_config(folder: str):
-    """(architecture, typed config) of a model folder."""
+    """(architecture, typed config) of a model folder.  A configuration class that says so (a static method
+    sizes_from_tensors(raw, shapes)) gets the shapes of the folder's tensors first, for sizes that its config.json leaves
+    to them; only the files' headers are read for that."""
     raw = read_config_json(folder)
     arch = architecture_for(raw)
+    complete = getattr(arch.config_cls, "sizes_from_tensors", None)
+    if complete is not None:
+        raw = complete(raw, tensor_shapes(folder))
     return arch, arch.config_cls.from_dict(raw)
+
+
+def tensor_shapes(folder: str) -> dict:
+    """name -> shape of every tensor in the folder's weight files ({} when there are none to read)."""
+    from ..weights.safetensors_io import SafetensorsError, open_model_files
+    try:
+        files = open_model_files(folder)
+    except SafetensorsError:
+        return {}
+    try:
+        return {n: tuple(f.entries[n][1]) for f in files for n in f.names()}
+    finally:
+        for f in files:
+            f.close()
 
 
 def _positive_int(raw: dict, key: str, default: Optional[int] = None) -> int:

@@ -41,6 +41,11 @@ struct AttnArgs {
                               // memory; the keys per split follow from it (bn_split_chunk) instead of from `chunk`
     int fold;                 // > 0: keys are summed in runs of `fold` positions (a multiple of BN_PAGE, counted from
                               // position 0) and the runs folded in order (fold_factors, fold_value below); a split is then one run
+    int vd;                   // width of a value head (the keys' hs unless the mixer says otherwise); out, part_o and the
+                              // value pages are vd wide
+    const float* dist_a;      // [H] or null: a bias that grows with the distance is taken off the score of query i and
+    const float* dist_b;      // key j: dist_a[h] * ln(1 + dist_b[h] * (i - j))
+    int sink;                 // 1: the softmax has one more term of score 0 and no value (1 is added to its denominator)
 };
 
 // The fold of one run of keys into the sums of the runs before it: (M, L, O) <- (M, L, O) + (m, l, o) with both sides
@@ -52,6 +57,15 @@ __device__ __forceinline__ void fold_factors(float M, float m, float& m2, float&
     fb = expf(m - m2);
 }
 __device__ __forceinline__ float fold_value(float O, float fa, float o, float fb) { return __fmaf_rn(O, fa, __fmul_rn(o, fb)); }
+
+// The sink of a softmax, as one more run of keys with maximum 0, sum 1 and no values, folded last with the operations of a
+// fold: every path (one workgroup, folded runs, merged splits) ends with the same step.
+__device__ __forceinline__ void fold_sink(float& M, float& L, float& fa) {
+    float m2, fb;
+    fold_factors(M, 0.f, m2, fa, fb);                    // fa = 0 when the row saw no key
+    L = fold_value(L, fa, 1.f, fb);
+    M = m2;
+}
 
 template <typename T> struct Vec4;
 template <> struct Vec4<float> {
@@ -73,8 +87,9 @@ template <> struct Vec4<bf16> {
 template <typename T, int RT>
 __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    const int hs = a.hs, KT = a.KT, GT = a.GT;
+    const int hs = a.hs, vd = a.vd, KT = a.KT, GT = a.GT;
     const int hsp = (hs + 7) & ~7;                       // the head size padded to whole groups of 8
+    const int vdp = (vd + 7) & ~7;
     const int QT = RT / GT;
     const int G = a.H / a.Hkv;
     const int n_head_tiles = (G + GT - 1) / GT;
@@ -94,6 +109,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
 
     // shared memory
     const int kstride = hsp + 16 / (int)sizeof(T);       // elements; keeps rows 16-byte aligned
+    const int vstride = vdp + 16 / (int)sizeof(T);
     float* q_s = reinterpret_cast<float*>(smem_raw);     // [RT][hsp], zero beyond hs
     float* s_s = q_s + RT * hsp;                         // [RT][KT] scores
     float* p_s = s_s + RT * KT;                          // [KT][RT] probabilities
@@ -122,8 +138,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     }
     if (tid < 16) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; Mt_s[tid] = -INFINITY; Lt_s[tid] = 0.f; }
     const bool whole_groups = (hs * (int)sizeof(T)) % 16 == 0;      // rows of 16-byte groups in the pages
-    if (hsp != hs)                                                  // the padding of the staged rows stays zero
-        for (int idx = tid; idx < 2 * KT * kstride; idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
+    const bool whole_groups_v = (vd * (int)sizeof(T)) % 16 == 0;
+    if (hsp != hs || vdp != vd)                                     // the padding of the staged rows stays zero
+        for (int idx = tid; idx < KT * (kstride + vstride); idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
 
     // keys this workgroup visits
     int lo = 0, hi = 0;
@@ -136,7 +153,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     }
 
     // phase C ownership: thread -> (jp, dp): keys jp, jp+JP, ...; output dims 2dp, 2dp+1
-    const int DP = hs / 2;
+    const int DP = vd / 2;
     int JP = ATT_THREADS / DP; if (JP > 8) JP = 8; if (JP > KT) JP = KT;
     const int jp = tid / DP, dp = tid - jp * DP;
     const bool c_active = jp < JP;
@@ -148,18 +165,18 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
     float tot[RT][2];
 #pragma unroll
     for (int r = 0; r < RT; ++r) { tot[r][0] = 0.f; tot[r][1] = 0.f; }
-    // Adds the JP partial accumulators up in a fixed order, through `scratch` ([RT][hs] floats that nobody else uses now);
+    // Adds the JP partial accumulators up in a fixed order, through `scratch` ([RT][vd] floats that nobody else uses now);
     // the threads with jp == 0 then hold the sums.
     auto sum_partials = [&](float* scratch) {
         for (int src = 1; src < JP; ++src) {
             if (c_active && jp == src) {
 #pragma unroll
-                for (int r = 0; r < RT; ++r) { scratch[r * hs + 2 * dp] = acc[r][0]; scratch[r * hs + 2 * dp + 1] = acc[r][1]; }
+                for (int r = 0; r < RT; ++r) { scratch[r * vd + 2 * dp] = acc[r][0]; scratch[r * vd + 2 * dp + 1] = acc[r][1]; }
             }
             __syncthreads();
             if (jp == 0) {
 #pragma unroll
-                for (int r = 0; r < RT; ++r) { acc[r][0] += scratch[r * hs + 2 * dp]; acc[r][1] += scratch[r * hs + 2 * dp + 1]; }
+                for (int r = 0; r < RT; ++r) { acc[r][0] += scratch[r * vd + 2 * dp]; acc[r][1] += scratch[r * vd + 2 * dp + 1]; }
             }
             __syncthreads();
         }
@@ -189,8 +206,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             }
             acc[r][0] = 0.f; acc[r][1] = 0.f;
         }
-        if (hsp != hs)                                    // the scratch lay over the staged rows, whose padding is zero
-            for (int idx = tid; idx < 2 * KT * kstride; idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
+        if (hsp != hs || vdp != vd)                       // the scratch lay over the staged rows, whose padding is zero
+            for (int idx = tid; idx < KT * (kstride + vstride); idx += ATT_THREADS) k_s[idx] = from_f32<T>(0.f);
         __syncthreads();
     };
 
@@ -204,34 +221,43 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         // ---- load the K and V tile (rows j0 .. j0+KT-1 of one page) ----
         {
             const int page = a.block_table[(size_t)seq * a.bt_stride + j0 / BN_PAGE];
-            const size_t base = (((size_t)page * a.Hkv + kvh) * BN_PAGE + (j0 % BN_PAGE)) * hs;
-            const int vec_per_row = hs * (int)sizeof(T) / 16;
+            const size_t prow = ((size_t)page * a.Hkv + kvh) * BN_PAGE + (j0 % BN_PAGE);
+            const size_t base = prow * hs, vbase = prow * vd;
+            const int vec_per_row = hs * (int)sizeof(T) / 16, vec_per_row_v = vd * (int)sizeof(T) / 16;
             const uint4* kg = reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(a.k_pages) + base);
-            const uint4* vg = reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(a.v_pages) + base);
+            const uint4* vg = reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(a.v_pages) + vbase);
             for (int idx = tid; whole_groups && idx < KT * vec_per_row; idx += ATT_THREADS) {
                 const int j = idx / vec_per_row, c = idx - j * vec_per_row;
-                uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-                if (j0 + j < hi) { kv = kg[idx]; if (!a.v_transposed) vv = vg[idx]; }   // rows not yet written stay zero
+                uint4 kv = make_uint4(0, 0, 0, 0);
+                if (j0 + j < hi) kv = kg[idx];                                          // rows not yet written stay zero
                 *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(k_s + j * kstride) + c * 16) = kv;
-                if (!a.v_transposed)
-                    *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(v_s + j * kstride) + c * 16) = vv;
+            }
+            for (int idx = tid; whole_groups_v && !a.v_transposed && idx < KT * vec_per_row_v; idx += ATT_THREADS) {
+                const int j = idx / vec_per_row_v, c = idx - j * vec_per_row_v;
+                uint4 vv = make_uint4(0, 0, 0, 0);
+                if (j0 + j < hi) vv = vg[idx];
+                *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(v_s + j * vstride) + c * 16) = vv;
             }
             if (!whole_groups) {
                 const T* ke = reinterpret_cast<const T*>(a.k_pages) + base;
-                const T* ve = reinterpret_cast<const T*>(a.v_pages) + base;
                 for (int idx = tid; idx < KT * hs; idx += ATT_THREADS) {
                     const int j = idx / hs, d = idx - j * hs;
-                    const bool in = j0 + j < hi;
-                    k_s[j * kstride + d] = in ? ke[idx] : from_f32<T>(0.f);
-                    if (!a.v_transposed) v_s[j * kstride + d] = in ? ve[idx] : from_f32<T>(0.f);
+                    k_s[j * kstride + d] = (j0 + j < hi) ? ke[idx] : from_f32<T>(0.f);
+                }
+            }
+            if (!whole_groups_v && !a.v_transposed) {
+                const T* ve = reinterpret_cast<const T*>(a.v_pages) + vbase;
+                for (int idx = tid; idx < KT * vd; idx += ATT_THREADS) {
+                    const int j = idx / vd, d = idx - j * vd;
+                    v_s[j * vstride + d] = (j0 + j < hi) ? ve[idx] : from_f32<T>(0.f);
                 }
             }
             if (a.v_transposed) {
-                const T* vt = reinterpret_cast<const T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * hs * BN_PAGE +
+                const T* vt = reinterpret_cast<const T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * vd * BN_PAGE +
                               (j0 % BN_PAGE);
-                for (int idx = tid; idx < KT * hs; idx += ATT_THREADS) {
+                for (int idx = tid; idx < KT * vd; idx += ATT_THREADS) {
                     const int d = idx / KT, j = idx - d * KT;
-                    v_s[j * kstride + d] = (j0 + j < hi) ? vt[(size_t)d * BN_PAGE + j] : from_f32<T>(0.f);
+                    v_s[j * vstride + d] = (j0 + j < hi) ? vt[(size_t)d * BN_PAGE + j] : from_f32<T>(0.f);
                 }
             }
         }
@@ -268,7 +294,12 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
                     const int qpos = pos0 + i;
                     bool ok = (i < n_tok) && (ht * GT + g < G) && key <= qpos && key >= lo && key < hi;
                     if (a.window > 0) ok = ok && (key > qpos - a.window);
-                    s_s[r * KT + ja] = ok ? dot[r] * a.scale : -INFINITY;
+                    float sc = dot[r] * a.scale;
+                    if (a.dist_a && ok) {
+                        const int head = kvh * G + ht * GT + g;
+                        sc -= a.dist_a[head] * logf(1.0f + a.dist_b[head] * (float)(qpos - key));
+                    }
+                    s_s[r * KT + ja] = ok ? sc : -INFINITY;
                 }
             }
         }
@@ -302,11 +333,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
                 float v0, v1;
                 if (sizeof(T) == 2) {
                     const uint32_t two = *reinterpret_cast<const uint32_t*>(
-                        reinterpret_cast<const unsigned char*>(v_s + j * kstride) + dp * 4);
+                        reinterpret_cast<const unsigned char*>(v_s + j * vstride) + dp * 4);
                     v0 = bf16lo_to_f32(two); v1 = bf16hi_to_f32(two);
                 } else {
                     const float2 two = *reinterpret_cast<const float2*>(
-                        reinterpret_cast<const unsigned char*>(v_s + j * kstride) + dp * 8);
+                        reinterpret_cast<const unsigned char*>(v_s + j * vstride) + dp * 8);
                     v0 = two.x; v1 = two.y;
                 }
 #pragma unroll
@@ -328,7 +359,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         fold_run();                                       // the last run; the result is in tot, Mt_s, Lt_s
     } else {
         // ---- sum the JP partial accumulators in a fixed order (q_s is free now) ----
-        sum_partials(q_s);
+        sum_partials(vd <= hsp ? q_s : reinterpret_cast<float*>(k_s));    // values wider than keys: the staged rows are free too
     }
     if (jp != 0) return;
 #pragma unroll
@@ -340,15 +371,21 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         const int head = kvh * G + hg;
         const size_t tok = (size_t)(tok0 + i);
         if (a.n_splits == 1) {
-            const float l = folded ? Lt_s[r] : l_s[r];
+            float l = folded ? Lt_s[r] : l_s[r];
+            float o0 = folded ? tot[r][0] : acc[r][0], o1 = folded ? tot[r][1] : acc[r][1];
+            if (a.sink) {
+                float m = folded ? Mt_s[r] : m_s[r], fa;
+                fold_sink(m, l, fa);
+                o0 = __fmul_rn(o0, fa); o1 = __fmul_rn(o1, fa);
+            }
             const float inv = l > 0.f ? 1.0f / l : 0.f;
-            T* o = reinterpret_cast<T*>(a.out) + tok * a.out_stride + (size_t)head * hs + 2 * dp;
-            o[0] = from_f32<T>(__fmul_rn(folded ? tot[r][0] : acc[r][0], inv));
-            o[1] = from_f32<T>(__fmul_rn(folded ? tot[r][1] : acc[r][1], inv));
+            T* o = reinterpret_cast<T*>(a.out) + tok * a.out_stride + (size_t)head * vd + 2 * dp;
+            o[0] = from_f32<T>(__fmul_rn(o0, inv));
+            o[1] = from_f32<T>(__fmul_rn(o1, inv));
         } else {
             const size_t row = (tok * a.H + head) * a.n_splits + split;
-            a.part_o[row * hs + 2 * dp] = acc[r][0];
-            a.part_o[row * hs + 2 * dp + 1] = acc[r][1];
+            a.part_o[row * vd + 2 * dp] = acc[r][0];
+            a.part_o[row * vd + 2 * dp + 1] = acc[r][1];
             if (dp == 0) { a.part_ml[row * 2] = m_s[r]; a.part_ml[row * 2 + 1] = l_s[r]; }
         }
     }
@@ -357,14 +394,14 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
 // out[row, d] = sum_s e^{m_s - m} o_s[d] / sum_s e^{m_s - m} l_s, splits in index order
 template <typename T>
 __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                    const float* __restrict__ part_ml, int H, int hs, int n_splits) {
-    const int row = blockIdx.x;               // token*H + head
+                                    const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink) {
+    const int row = blockIdx.x;               // token*H + head; hs: the width of a value head
     const int tok = row / H, head = row - tok * H;
     const float* ml = part_ml + (size_t)row * n_splits * 2;
-    float m = -INFINITY;
+    float m = sink ? 0.f : -INFINITY;
     for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
     for (int d = threadIdx.x; d < hs; d += blockDim.x) {
-        float num = 0.f, den = 0.f;
+        float num = 0.f, den = sink ? expf(-m) : 0.f;
         if (m != -INFINITY) {
             for (int s = 0; s < n_splits; ++s) {
                 const float w = expf(ml[2 * s] - m);          // 0 for an empty split
@@ -380,8 +417,8 @@ __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const f
 // operations of fold_factors and fold_value, which is what a workgroup that walks all runs by itself does; runs without keys are passed over.
 template <typename T>
 __global__ void attn_fold_kernel(T* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                 const float* __restrict__ part_ml, int H, int hs, int n_splits) {
-    const int row = blockIdx.x;               // token*H + head
+                                 const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink) {
+    const int row = blockIdx.x;               // token*H + head; hs: the width of a value head
     const int tok = row / H, head = row - tok * H;
     const float* ml = part_ml + (size_t)row * n_splits * 2;
     for (int d = threadIdx.x; d < hs; d += blockDim.x) {
@@ -395,21 +432,26 @@ __global__ void attn_fold_kernel(T* __restrict__ out, int out_stride, const floa
             O = fold_value(O, fa, part_o[((size_t)row * n_splits + s) * hs + d], fb);
             M = m2;
         }
+        if (sink) { float fa; fold_sink(M, L, fa); O = __fmul_rn(O, fa); }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         out[(size_t)tok * out_stride + (size_t)head * hs + d] = from_f32<T>(__fmul_rn(O, inv));
     }
 }
 
-static size_t attn_smem_bytes(int RT, int hs, int KT, int elt) {
-    const int hsp = (hs + 7) & ~7;
-    return (size_t)(RT * hsp + 2 * RT * KT + 112) * sizeof(float) + (size_t)2 * KT * (hsp * elt + 16);
+// vd: the width of a value head.  The staged keys and values double as the scratch of the partial accumulators' sum
+// ([RT][vd] floats); where values wider than keys make that too small, the shared memory is rounded up to it.
+static size_t attn_smem_bytes(int RT, int hs, int vd, int KT, int elt) {
+    const int hsp = (hs + 7) & ~7, vdp = (vd + 7) & ~7;
+    size_t staged = (size_t)KT * ((hsp + vdp) * elt + 32);
+    if (staged < (size_t)RT * vd * sizeof(float)) staged = (size_t)RT * vd * sizeof(float);
+    return (size_t)(RT * hsp + 2 * RT * KT + 112) * sizeof(float) + staged;
 }
 
 template <typename T, int RT>
 static int launch_rows(const AttnArgs& a, int n_tiles, hipStream_t s) {
     const int G = a.H / a.Hkv;
     const int n_head_tiles = (G + a.GT - 1) / a.GT;
-    const size_t smem = attn_smem_bytes(RT, a.hs, a.KT, (int)sizeof(T));
+    const size_t smem = attn_smem_bytes(RT, a.hs, a.vd, a.KT, (int)sizeof(T));
     hipLaunchKernelGGL((attn_rows_kernel<T, RT>), dim3(n_tiles, a.Hkv * n_head_tiles, a.n_splits),
                        dim3(ATT_THREADS), smem, s, a);
     return bn_launch_status();
@@ -432,12 +474,13 @@ static int launch_rows_rt(const AttnArgs& a, int RT, int n_tiles, hipStream_t s)
 // never of the rows a launch happens to hold: a query's keys are then cut into the same tiles, and
 // its sums formed in the same order, whether it arrives alone, in a prompt or in a batch (the
 // reference keeps one order per kernel, src/transformer/gqa_scalar.c:61-121).
-extern "C" int bn_attn_rows_key_tile(int dtype, int hs) {
+static int attn_key_tile(int dtype, int hs, int vd) {
     const int elt = dtype == BN_DT_F32 ? 4 : 2;
     for (int kt = 64; kt >= 16; kt >>= 1)
-        if (attn_smem_bytes(16, hs, kt, elt) <= 64 * 1024) return kt;
+        if (attn_smem_bytes(16, hs, vd, kt, elt) <= 64 * 1024) return kt;
     return 0;
 }
+extern "C" int bn_attn_rows_key_tile(int dtype, int hs) { return attn_key_tile(dtype, hs, hs); }
 
 // RT rows per workgroup = QT query tokens x GT heads.  tiles == null: decode (one token per
 // sequence, n_tiles sequences).  With n_splits > 1 the partial buffers must hold
@@ -447,7 +490,10 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             int bt_stride, const int* seq_lens, const int* tiles, int n_tiles,
                             int n_tokens, int H, int Hkv, int hs, int RT, int GT, int window,
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
-                            int v_transposed, const int* max_len, int fold, hipStream_t s) {
+                            int v_transposed, const int* max_len, int fold, int vd, const float* dist_a,
+                            const float* dist_b, int sink, hipStream_t s) {
+    if (vd == 0) vd = hs;
+    if (vd < 2 || vd > BN_MAX_HEAD_DIM || vd % 2 || (dist_a == nullptr) != (dist_b == nullptr)) return BN_ERR_ARG;
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
     // fold mode: runs of whole pages; a split is one run, and the runs' length does not follow the longest sequence
     if (fold < 0 || fold % BN_PAGE || (fold > 0 && n_splits > 1 && (chunk != fold || max_len))) return BN_ERR_ARG;
@@ -468,7 +514,8 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     a.scale = scale;
     a.v_transposed = v_transposed;
     a.fold = fold;
-    a.KT = bn_attn_rows_key_tile(dtype, hs);
+    a.vd = vd; a.dist_a = dist_a; a.dist_b = dist_b; a.sink = sink ? 1 : 0;
+    a.KT = attn_key_tile(dtype, hs, vd);
     if (a.KT == 0) return BN_ERR_ARG;
     int rc;
     if (dtype == BN_DT_F32) rc = launch_rows_rt<float>(a, RT, n_tiles, s);
@@ -478,17 +525,17 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     if (fold > 0) {
         if (dtype == BN_DT_F32)
             hipLaunchKernelGGL(attn_fold_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out, out_stride, part_o,
-                               part_ml, H, hs, n_splits);
+                               part_ml, H, vd, n_splits, a.sink);
         else
             hipLaunchKernelGGL(attn_fold_kernel<bf16>, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
-                               part_ml, H, hs, n_splits);
+                               part_ml, H, vd, n_splits, a.sink);
         return bn_launch_status();
     }
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(attn_combine_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out,
-                           out_stride, part_o, part_ml, H, hs, n_splits);
+                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink);
     else
         hipLaunchKernelGGL(attn_combine_kernel<bf16>, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out,
-                           out_stride, part_o, part_ml, H, hs, n_splits);
+                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink);
     return bn_launch_status();
 }

@@ -139,4 +139,24 @@ __device__ __forceinline__ float bn_gate_act(float g, int act) {
     return p * p;
 }
 
+// Activations of one argument (a feed-forward without a gate; the inner layer of a low-rank projection).
+// The Python side reads these lines.
+#define BN_UNARY_GELU_ERF 0      // 0.5 z (1 + erf(z / sqrt 2))
+#define BN_UNARY_GELU_TANH 1     // the tanh form, as bn_gate_act's
+#define BN_UNARY_SILU 2
+#define BN_UNARY_RELU2 3
+#define BN_UNARY_TANH 4
+#define BN_UNARY_SIGMOID 5
+#define BN_UNARY_KINDS 6
+__device__ __forceinline__ float bn_unary_act(float z, int kind) {
+    switch (kind) {
+        case BN_UNARY_GELU_ERF: return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+        case BN_UNARY_GELU_TANH: return bn_gate_act(z, BN_ACT_GELU_TANH);
+        case BN_UNARY_SILU: return bn_gate_act(z, BN_ACT_SILU);
+        case BN_UNARY_RELU2: return bn_gate_act(z, BN_ACT_RELU2);
+        case BN_UNARY_TANH: return tanhf(z);
+        default: return 1.0f / (1.0f + expf(-z));
+    }
+}
+
 static inline int bn_launch_status() { return (int)hipGetLastError(); }

@@ -497,3 +497,131 @@ extern "C" int bn_bias_add(int dtype, void* y, const float* b, int n_rows, int N
         return BN_ERR_DTYPE;
     return bn_launch_status();
 }
+
+// ---- an embedding with a sinusoidal position vector -------------------------------------------------------------
+// x[t, e] = table[token, e] * scale + (e even ? sin : cos)(position * freq[e / 2]); position, angle, sine and cosine in
+// float32 (the accurate functions, with their range reduction).  A row without a position (< 0: padding) gets none.
+template <typename T>
+__global__ void embed_gather_sinusoid_kernel(float* __restrict__ x, const T* __restrict__ table,
+                                             const int* __restrict__ tokens, const int* __restrict__ positions,
+                                             const float* __restrict__ freq, int dim, int vocab, float scale) {
+    const int t = blockIdx.x;
+    const int tok = tokens[t], pos = positions[t];
+    float* row = x + (size_t)t * dim;
+    const bool known = tok >= 0 && tok < vocab;
+    const T* src = table + (size_t)(known ? tok : 0) * dim;
+    for (int e = threadIdx.x; e < dim; e += blockDim.x) {
+        float v = known ? to_f32(src[e]) * scale : 0.f;
+        if (pos >= 0) {
+            const float angle = __fmul_rn((float)pos, freq[e >> 1]);
+            v += (e & 1) ? cosf(angle) : sinf(angle);
+        }
+        row[e] = v;
+    }
+}
+
+extern "C" int bn_embed_gather_sinusoid(int dtype, void* x, const void* table, const int* tokens, const int* positions,
+                                        const float* freq, int n_tokens, int dim, int vocab, float scale, hipStream_t s) {
+    if (n_tokens <= 0 || dim <= 0 || vocab <= 0 || !positions || !freq) return BN_ERR_ARG;
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(embed_gather_sinusoid_kernel<float>, dim3(n_tokens), dim3(256), 0, s, (float*)x, (const float*)table,
+                           tokens, positions, freq, dim, vocab, scale);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(embed_gather_sinusoid_kernel<bf16>, dim3(n_tokens), dim3(256), 0, s, (float*)x, (const bf16*)table,
+                           tokens, positions, freq, dim, vocab, scale);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- activations of one argument (bn_unary_act of common.h) over a tensor ----------------------------------------
+template <typename T>
+__global__ void unary_act_kernel(T* __restrict__ out, const T* __restrict__ in, size_t n, int kind) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = from_f32<T>(bn_unary_act(to_f32(in[i]), kind));
+}
+
+// eight bf16 values a thread
+__global__ void unary_act_bf16x8_kernel(bf16* __restrict__ out, const bf16* __restrict__ in, size_t n8, int kind) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const uint4 v = reinterpret_cast<const uint4*>(in)[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const bf16 lo = from_f32<bf16>(bn_unary_act(bf16lo_to_f32(w[k]), kind));
+        const bf16 hi = from_f32<bf16>(bn_unary_act(bf16hi_to_f32(w[k]), kind));
+        o[k] = (uint32_t)(*reinterpret_cast<const uint16_t*>(&lo)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&hi)) << 16);
+    }
+    reinterpret_cast<uint4*>(out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+extern "C" int bn_unary_act_apply(int dtype, void* out, const void* in, long long n, int kind, hipStream_t s) {
+    if (n <= 0 || kind < 0 || kind >= BN_UNARY_KINDS || !out || !in) return BN_ERR_ARG;
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(unary_act_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (float*)out,
+                           (const float*)in, (size_t)n, kind);
+    else if (dtype == BN_DT_BF16 && n % 8 == 0 && !(((uintptr_t)out | (uintptr_t)in) & 15))
+        hipLaunchKernelGGL(unary_act_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, (bf16*)out,
+                           (const bf16*)in, (size_t)(n / 8), kind);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(unary_act_kernel<bf16>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (bf16*)out,
+                           (const bf16*)in, (size_t)n, kind);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// logits times a constant of the architecture, in place
+__global__ void scale_kernel(float* __restrict__ x, size_t n, float f) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] *= f;
+}
+
+extern "C" int bn_scale(float* x, long long n, float f, hipStream_t s) {
+    if (n <= 0 || !x) return BN_ERR_ARG;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, (size_t)n, f);
+    return bn_launch_status();
+}
+
+// ---- the mean of several branches, each under an RMSNorm of its own --------------------------------------------------
+// out[r] = (1 / n) sum_b  in_b[r] / sqrt(mean(in_b[r]^2) + eps) * w_b      (n = 1 or 2 branches; float32 sums)
+template <typename T>
+__global__ void rmsnorm_mean_kernel(T* __restrict__ out, const T* __restrict__ a, const T* __restrict__ b,
+                                    const float* __restrict__ wa, const float* __restrict__ wb, int dim, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const T* ra = a + (size_t)r * dim;
+    const T* rb = b ? b + (size_t)r * dim : nullptr;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float va = to_f32(ra[i]);
+        sa = fmaf(va, va, sa);
+        if (rb) { const float vb = to_f32(rb[i]); sb = fmaf(vb, vb, sb); }
+    }
+    sa = block_sum(sa, scratch);
+    const float fa = 1.0f / sqrtf(sa / (float)dim + eps);
+    float fb = 0.f;
+    if (rb) { sb = block_sum(sb, scratch); fb = 1.0f / sqrtf(sb / (float)dim + eps); }
+    const float share = rb ? 0.5f : 1.0f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        float v = to_f32(ra[i]) * fa * wa[i];
+        if (rb) v += to_f32(rb[i]) * fb * wb[i];
+        out[(size_t)r * dim + i] = from_f32<T>(v * share);
+    }
+}
+
+extern "C" int bn_rmsnorm_mean(int dtype, void* out, const void* a, const void* b, const float* wa, const float* wb,
+                               int n_rows, int dim, float eps, hipStream_t s) {
+    if (n_rows <= 0 || dim <= 0 || !out || !a || !wa || (b && !wb)) return BN_ERR_ARG;
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(rmsnorm_mean_kernel<float>, dim3(n_rows), dim3(256), 0, s, (float*)out, (const float*)a,
+                           (const float*)b, wa, wb, dim, eps);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(rmsnorm_mean_kernel<bf16>, dim3(n_rows), dim3(256), 0, s, (bf16*)out, (const bf16*)a,
+                           (const bf16*)b, wa, wb, dim, eps);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}

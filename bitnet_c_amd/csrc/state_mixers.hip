@@ -1,0 +1,285 @@
+// Mixers that carry a state of fixed size from token to token instead of keys and values: the kernels of their
+// recurrences, for prompt and decode steps alike.  Every state lives in float32 in the cache's state area, a row per
+// sequence slot; a kernel finds a sequence's row through the step's device-side slot ids and its tokens either through
+// a list of tiles (one tile a sequence: sequence, first row, rows, position of the first; a tile of no rows is skipped)
+// or, tiles == null, as row b = the one new token of sequence b (seq_lens[b] == 0: a padding row, nothing is touched).
+// Everything that enters a recurrence is float32: decays, gates, exponentials, the state; the projections that feed
+// them arrive in the activations' type.  The order of every sum is a function of the sizes alone.
+//
+//   token shift   mix_s[t] = h[t] + (h[t-1] - h[t]) * mu_s; h[-1] of a step is the state's copy of the last h, 0 at position 0
+//   wkv           o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T;  w_t = exp(-exp(d_t + w0))   per head
+//   head norm     y = o / sqrt(mean_head(o^2) + eps) * weight * silu(gate)
+//   min-GRU       z = sigmoid(a + bz); c = b + bx; cand = c >= 0 ? c + 1/2 : sigmoid(c); S <- (1 - z) S + z cand; y = S silu(g)
+#include "common.h"
+#include <math.h>
+
+struct SeqRange { int seq, row0, n, pos0; };
+
+__device__ __forceinline__ SeqRange seq_range(const int* tiles, const int* seq_lens, int idx) {
+    SeqRange r;
+    if (tiles) {
+        const int* t = tiles + 4 * idx;
+        r.seq = t[0]; r.row0 = t[1]; r.n = t[2]; r.pos0 = t[3];
+    } else {
+        r.seq = idx; r.row0 = idx; r.pos0 = seq_lens[idx] - 1; r.n = r.pos0 >= 0 ? 1 : 0;
+    }
+    return r;
+}
+
+// ---- token shift ----------------------------------------------------------------------------------------------------
+// out[s, t, :] for s < n_mix.  The previous row of the flattened batch is the previous token when it belongs to the same
+// sequence; else the sequence's state holds it (zero at position 0).  The state is read only: the recurrence's
+// kernel stores the step's last h afterwards, when every reader is done.
+template <typename T>
+__global__ void token_shift_kernel(T* __restrict__ out, const T* __restrict__ h, const float* __restrict__ mu,
+                                   const float* __restrict__ state, size_t state_stride, const int* __restrict__ positions,
+                                   const int* __restrict__ seq_index, const int* __restrict__ slot_ids, int T_rows, int D,
+                                   int n_mix) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    const T* cur = h + (size_t)t * D;
+    const bool inside = t > 0 && pos > 0 && seq_index[t - 1] == seq_index[t] && positions[t - 1] == pos - 1;
+    const T* prev_row = inside ? h + (size_t)(t - 1) * D : nullptr;
+    const float* prev_state = (!inside && pos > 0) ? state + (size_t)slot_ids[seq_index[t]] * state_stride : nullptr;
+    for (int e = threadIdx.x; e < D; e += blockDim.x) {
+        const float c = to_f32(cur[e]);
+        const float p = prev_row ? to_f32(prev_row[e]) : (prev_state ? prev_state[e] : 0.f);
+        const float d = p - c;
+        for (int s = 0; s < n_mix; ++s)
+            out[((size_t)s * T_rows + t) * D + e] = from_f32<T>(pos >= 0 ? fmaf(d, mu[(size_t)s * D + e], c) : 0.f);
+    }
+}
+
+extern "C" int bn_token_shift(int dtype, void* out, const void* h, const float* mu, const float* state,
+                              long long state_stride, const int* positions, const int* seq_index, const int* slot_ids,
+                              int n_tokens, int D, int n_mix, hipStream_t s) {
+    if (n_tokens <= 0 || D <= 0 || n_mix <= 0 || !out || !h || !mu || !state || !positions || !seq_index || !slot_ids)
+        return BN_ERR_ARG;
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(token_shift_kernel<float>, dim3(n_tokens), dim3(256), 0, s, (float*)out, (const float*)h, mu, state,
+                           (size_t)state_stride, positions, seq_index, slot_ids, n_tokens, D, n_mix);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(token_shift_kernel<bf16>, dim3(n_tokens), dim3(256), 0, s, (bf16*)out, (const bf16*)h, mu, state,
+                           (size_t)state_stride, positions, seq_index, slot_ids, n_tokens, D, n_mix);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- the wkv recurrence -----------------------------------------------------------------------------------------------
+// A workgroup owns (sequence, head, a block of CB value columns).  Column j of a head's state S[dk, dv] depends on no
+// other column, so the columns are spread over threads and workgroups freely; the dk rows of a column are spread over
+// P threads (P a power of two <= 64, neighbouring lanes), each holding up to WKV_KR rows in registers, row i = p + P ii.
+// The tokens of a sequence come in chunks of TC: r, k, the decay and the block's v are staged in shared memory once a
+// chunk (rows beyond dk zero, which leaves the unused registers zero), then the chunk's tokens run without a barrier.
+#define WKV_KR 16
+#define WKV_MAX_DIM 256
+
+struct WkvArgs {
+    const void* r; const void* k; const void* v; const void* d;     // [T, ld*]: head h at h * dk (v: h * dv)
+    int ldr, ldk, ldv, ldd;
+    const float* w0;          // [H * dk] added to d before the exponentials
+    const float* u;           // [H * dk] the bonus of the current token
+    float* o;                 // [T, H * dv] float32
+    const void* h;            // [T, D]: the mixer's input, whose last row of every sequence becomes the state's copy
+    float* state;             // [slots, state_stride]: S as [H][dk][dv], then D values of the last h
+    size_t state_stride;
+    const int* tiles; const int* seq_lens; const int* slot_ids;
+    int H, dk, dv, D, P, CB, TC;
+};
+
+template <typename T>
+__global__ void wkv_scan_kernel(WkvArgs a) {
+    extern __shared__ float smem[];
+    const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
+    if (sr.n <= 0 || sr.pos0 < 0) return;
+    const int head = blockIdx.y, cb = blockIdx.z;
+    const int P = a.P, dk = a.dk, dv = a.dv, TC = a.TC;
+    const int dkp = P * WKV_KR;                           // staged rows, zero beyond dk
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int p = tid % P, jl = tid / P;
+    const int j = cb * a.CB + jl;                         // this thread's value column
+    const bool owns = jl < a.CB && j < dv;
+    float* r_s = smem;                                    // [TC][dkp]
+    float* k_s = r_s + TC * dkp;
+    float* w_s = k_s + TC * dkp;
+    float* v_s = w_s + TC * dkp;                          // [TC][CB]
+
+    float* S_g = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * dk * dv;
+    float S[WKV_KR], ub[WKV_KR];
+#pragma unroll
+    for (int ii = 0; ii < WKV_KR; ++ii) {
+        const int i = p + P * ii;
+        const bool in = owns && i < dk;
+        S[ii] = (in && sr.pos0 > 0) ? S_g[(size_t)i * dv + j] : 0.f;
+        ub[ii] = (in) ? a.u[(size_t)head * dk + i] : 0.f;
+    }
+
+    for (int c0 = 0; c0 < sr.n; c0 += TC) {
+        const int nc = min(TC, sr.n - c0);
+        __syncthreads();                                  // the chunk before this one has been consumed
+        for (int idx = tid; idx < nc * dkp; idx += nthreads) {
+            const int tt = idx / dkp, i = idx - tt * dkp;
+            const size_t row = (size_t)(sr.row0 + c0 + tt);
+            float rv = 0.f, kv = 0.f, wv = 0.f;
+            if (i < dk) {
+                const size_t c = (size_t)head * dk + i;
+                rv = to_f32(reinterpret_cast<const T*>(a.r)[row * a.ldr + c]);
+                kv = to_f32(reinterpret_cast<const T*>(a.k)[row * a.ldk + c]);
+                wv = expf(-expf(to_f32(reinterpret_cast<const T*>(a.d)[row * a.ldd + c]) + a.w0[c]));
+            }
+            r_s[idx] = rv; k_s[idx] = kv; w_s[idx] = wv;
+        }
+        for (int idx = tid; idx < nc * a.CB; idx += nthreads) {
+            const int tt = idx / a.CB, c = idx - tt * a.CB;
+            const int col = cb * a.CB + c;
+            v_s[idx] = col < dv ? to_f32(reinterpret_cast<const T*>(a.v)[(size_t)(sr.row0 + c0 + tt) * a.ldv +
+                                                                          (size_t)head * dv + col]) : 0.f;
+        }
+        __syncthreads();
+        if (jl < a.CB) {
+            for (int tt = 0; tt < nc; ++tt) {
+                const float vj = v_s[tt * a.CB + jl];
+                const float* rr = r_s + tt * dkp + p;
+                const float* kk = k_s + tt * dkp + p;
+                const float* ww = w_s + tt * dkp + p;
+                float acc = 0.f;
+#pragma unroll
+                for (int ii = 0; ii < WKV_KR; ++ii) {
+                    const float kv = kk[P * ii] * vj;
+                    acc = fmaf(rr[P * ii], fmaf(ub[ii], kv, S[ii]), acc);
+                    S[ii] = fmaf(ww[P * ii], S[ii], kv);
+                }
+                for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, BN_WAVE);
+                if (p == 0 && owns) a.o[(size_t)(sr.row0 + c0 + tt) * (a.H * dv) + (size_t)head * dv + j] = acc;
+            }
+        }
+    }
+#pragma unroll
+    for (int ii = 0; ii < WKV_KR; ++ii) {
+        const int i = p + P * ii;
+        if (owns && i < dk) S_g[(size_t)i * dv + j] = S[ii];
+    }
+    if (head == 0 && cb == 0) {                           // the step's last h of this sequence, for the next step's shift
+        float* hp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)a.H * dk * dv;
+        const T* last = reinterpret_cast<const T*>(a.h) + (size_t)(sr.row0 + sr.n - 1) * a.D;
+        for (int e = tid; e < a.D; e += nthreads) hp[e] = to_f32(last[e]);
+    }
+}
+
+// The split of a head over threads and workgroups, as the launch below makes it (P, CB, TC, threads): the host side
+// asks for it to size nothing, only to say which head sizes are taken.
+static bool wkv_shape(int dk, int dv, int& P, int& CB, int& TC, int& threads) {
+    if (dk < 1 || dv < 1 || dk > WKV_MAX_DIM || dv > WKV_MAX_DIM) return false;
+    P = 1;
+    while (P * WKV_KR < dk) P <<= 1;                      // <= 16
+    CB = dv < 256 / P ? dv : 256 / P;
+    threads = ((CB * P + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
+    TC = P * WKV_KR <= 128 ? 16 : 8;
+    return true;
+}
+
+extern "C" int bn_wkv_supports(int dk, int dv) {
+    int P, CB, TC, th;
+    return wkv_shape(dk, dv, P, CB, TC, th) ? 1 : 0;
+}
+
+extern "C" int bn_wkv_scan(int dtype, const void* r, int ldr, const void* k, int ldk, const void* v, int ldv, const void* d,
+                           int ldd, const float* w0, const float* u, float* o, const void* h, float* state,
+                           long long state_stride, const int* tiles, int n_tiles, const int* seq_lens, const int* slot_ids,
+                           int H, int dk, int dv, int D, hipStream_t s) {
+    WkvArgs a;
+    int threads;
+    if (!wkv_shape(dk, dv, a.P, a.CB, a.TC, threads) || n_tiles <= 0 || H <= 0 || D <= 0) return BN_ERR_ARG;
+    if (!r || !k || !v || !d || !w0 || !u || !o || !h || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
+    if (state_stride < (long long)H * dk * dv + D) return BN_ERR_ARG;
+    a.r = r; a.k = k; a.v = v; a.d = d; a.ldr = ldr; a.ldk = ldk; a.ldv = ldv; a.ldd = ldd;
+    a.w0 = w0; a.u = u; a.o = o; a.h = h; a.state = state; a.state_stride = (size_t)state_stride;
+    a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;
+    a.H = H; a.dk = dk; a.dv = dv; a.D = D;
+    const size_t smem = (size_t)a.TC * (3 * a.P * WKV_KR + a.CB) * sizeof(float);
+    const dim3 grid(n_tiles, H, (dv + a.CB - 1) / a.CB);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(wkv_scan_kernel<float>, grid, dim3(threads), smem, s, a);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(wkv_scan_kernel<bf16>, grid, dim3(threads), smem, s, a);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- per-head RMS of the recurrence's output, its weight and the gate -----------------------------------------------
+// one wave per (row, head): y = o / sqrt(mean(o^2) + eps) * weight * silu(gate)
+template <typename T>
+__global__ __launch_bounds__(BN_WAVE) void head_norm_gate_kernel(T* __restrict__ y, const float* __restrict__ o,
+                                                                  const T* __restrict__ gate, int ldg,
+                                                                  const float* __restrict__ weight, int H, int dv, float eps) {
+    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const float* ov = o + ((size_t)t * H + head) * dv;
+    float ss = 0.f;
+    for (int e = lane; e < dv; e += BN_WAVE) ss = fmaf(ov[e], ov[e], ss);
+    ss = wave_sum(ss);
+    const float f = 1.0f / sqrtf(ss / (float)dv + eps);
+    for (int e = lane; e < dv; e += BN_WAVE) {
+        const float g = to_f32(gate[(size_t)t * ldg + (size_t)head * dv + e]);
+        y[((size_t)t * H + head) * dv + e] = from_f32<T>(ov[e] * f * weight[(size_t)head * dv + e] * bn_unary_act(g, BN_UNARY_SILU));
+    }
+}
+
+extern "C" int bn_head_norm_gate(int dtype, void* y, const float* o, const void* gate, int ldg, const float* weight,
+                                 int n_tokens, int H, int dv, float eps, hipStream_t s) {
+    if (n_tokens <= 0 || H <= 0 || dv <= 0 || !y || !o || !gate || !weight || ldg < H * dv) return BN_ERR_ARG;
+    const dim3 grid(n_tokens, H);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, dim3(BN_WAVE), 0, s, (float*)y, o, (const float*)gate, ldg, weight, H, dv, eps);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(head_norm_gate_kernel<bf16>, grid, dim3(BN_WAVE), 0, s, (bf16*)y, o, (const bf16*)gate, ldg, weight, H, dv, eps);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- min-GRU ------------------------------------------------------------------------------------------------------
+// zxg [T, ld]: the three projections side by side (update gate at 0, candidate at W, output gate at 2 W), without their
+// biases; a thread owns one channel of one sequence and walks its tokens.
+template <typename T>
+__global__ void mingru_scan_kernel(T* __restrict__ y, const T* __restrict__ zxg, int ld, const float* __restrict__ bz,
+                                   const float* __restrict__ bx, float* __restrict__ state, size_t state_stride,
+                                   const int* __restrict__ tiles, const int* __restrict__ seq_lens,
+                                   const int* __restrict__ slot_ids, int W) {
+    const SeqRange sr = seq_range(tiles, seq_lens, blockIdx.x);
+    if (sr.n <= 0 || sr.pos0 < 0) return;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= W) return;
+    float* sp = state + (size_t)slot_ids[sr.seq] * state_stride + c;
+    float S = sr.pos0 > 0 ? *sp : 0.f;
+    const float biasz = bz ? bz[c] : 0.f, biasx = bx ? bx[c] : 0.f;
+    const T* in = zxg + (size_t)sr.row0 * ld + c;
+    T* out = y + (size_t)sr.row0 * W + c;
+#pragma unroll 4
+    for (int t = 0; t < sr.n; ++t) {
+        const float zp = to_f32(in[(size_t)t * ld]) + biasz;
+        const float cp = to_f32(in[(size_t)t * ld + W]) + biasx;
+        const float g = to_f32(in[(size_t)t * ld + 2 * W]);
+        const float z = 1.0f / (1.0f + expf(-zp));
+        const float cand = cp >= 0.f ? cp + 0.5f : 1.0f / (1.0f + expf(-cp));
+        S = fmaf(z, cand - S, S);                         // (1 - z) S + z cand
+        out[(size_t)t * W] = from_f32<T>(S * bn_unary_act(g, BN_UNARY_SILU));
+    }
+    *sp = S;
+}
+
+extern "C" int bn_mingru_scan(int dtype, void* y, const void* zxg, int ld, const float* bz, const float* bx, float* state,
+                              long long state_stride, const int* tiles, int n_tiles, const int* seq_lens,
+                              const int* slot_ids, int W, hipStream_t s) {
+    if (n_tiles <= 0 || W <= 0 || ld < 3 * W || !y || !zxg || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
+    if (state_stride < W) return BN_ERR_ARG;
+    const int threads = W >= 256 ? 256 : ((W + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
+    const dim3 grid(n_tiles, (W + threads - 1) / threads);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(mingru_scan_kernel<float>, grid, dim3(threads), 0, s, (float*)y, (const float*)zxg, ld, bz, bx, state,
+                           (size_t)state_stride, tiles, seq_lens, slot_ids, W);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(mingru_scan_kernel<bf16>, grid, dim3(threads), 0, s, (bf16*)y, (const bf16*)zxg, ld, bz, bx, state,
+                           (size_t)state_stride, tiles, seq_lens, slot_ids, W);
+    else
+        return BN_ERR_DTYPE;
+    return bn_launch_status();
+}

@@ -47,6 +47,7 @@ class DecoderModel:
         self.blocks = [BLOCKS.build(lp.block) for lp in plan.layers]
         self.final_norm = NORMS.build(plan.final_norm) if plan.final_norm is not None else None
         self.lm_head_bias = None         # [V] float32, when the plan names one
+        self.position_freq = None        # [ceil(D / 2)] float32: the frequencies of a sinusoidal position vector, when the plan has one
         self.embedding = None            # [V, D] in the compute dtype
         self.lm_head = None              # [V, D]; the embedding itself when tied
 
@@ -67,6 +68,8 @@ class DecoderModel:
         if p.lm_head_bias_name is not None:
             self.lm_head_bias = upload(tensors[p.lm_head_bias_name], self.device, torch.float32)
             done([p.lm_head_bias_name])
+        if p.position_sinusoid_base > 0:
+            self.position_freq = ops.sinusoid_frequencies(p.hidden_size, p.position_sinusoid_base).to(self.device)
         self.embedding = upload(tensors[p.embedding_name], self.device, self.dtype)
         done([p.embedding_name])
         if p.lm_head_name is None:
@@ -169,7 +172,11 @@ class DecoderModel:
     def forward(self, ctx, views) -> torch.Tensor:
         """ctx: the step's StepContext; views[i]: the KVView of schedule entry i.
         Returns float32 logits [len(ctx.want_rows), vocab]."""
-        x = ops.embed_gather(self.embedding, ctx.tokens, self.plan.embedding_multiplier)    # src/model_embed.c:6-28
+        if self.position_freq is not None:
+            x = ops.embed_gather_sinusoid(self.embedding, ctx.tokens, ctx.positions, self.position_freq,
+                                          self.plan.embedding_multiplier)
+        else:
+            x = ops.embed_gather(self.embedding, ctx.tokens, self.plan.embedding_multiplier)    # src/model_embed.c:6-28
         stream = ResidualStream(x)
         for i, e in enumerate(self.plan.schedule):
             ctx.entry = i
@@ -180,6 +187,8 @@ class DecoderModel:
         else:
             h = ops.gather_rows(stream.flush(), ctx.want_rows, self.dtype)
         logits = ops.linear(h, self.lm_head, torch.float32, streamed=self.head.streamed)
+        if self.plan.logit_scale != 1.0:
+            ops.scale_(logits, self.plan.logit_scale)
         if self.lm_head_bias is not None and logits.shape[0]:
             ops.bias_add(logits, self.lm_head_bias)
         if self.plan.logit_softcap > 0:                            # src/transformer/logits.c:325-333

@@ -46,10 +46,17 @@ class ModelPlan:
     embedding_multiplier: float = 1.0    # the embedding row times this before the first block
     logit_softcap: float = 0.0           # > 0: logits = cap * tanh(logits / cap)
     lm_head_bias_name: Optional[str] = None   # a bias [vocab] added to the logits (before the soft-cap); None: none
+    # Positions that enter with the embedding instead of inside the mixers: > 0 adds a sinusoidal vector to every
+    # embedding row, entry 2i = sin(p base^(-2i/hidden)), entry 2i + 1 = cos of the same angle.
+    position_sinusoid_base: float = 0.0
+    logit_scale: float = 1.0             # the logits times this (before a bias or a soft-cap)
 
     def validate(self) -> None:
         if not self.embedding_multiplier > 0 or self.logit_softcap < 0:
             raise ValueError("the embedding multiplier must be positive and the logit soft-cap 0 (none) or positive")
+        if self.position_sinusoid_base < 0 or self.position_sinusoid_base == 1 or not self.logit_scale > 0:
+            raise ValueError("the base of a sinusoidal position vector is 0 (none) or a positive number other than 1, "
+                             "and the logits' multiplier is positive")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"schedule entry {i} names layer {e.layer}; there are {len(self.layers)}")

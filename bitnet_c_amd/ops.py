@@ -44,6 +44,26 @@ _SIGNATURES = {
         "bn_sum_deferred": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "bn_swiglu_scaled": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
         "bn_bias_add": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "bn_embed_gather_sinusoid": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
+                                     c_void_p],
+        "bn_unary_act_apply": [c_int, c_void_p, c_void_p, c_longlong, c_int, c_void_p],
+        "bn_scale": [c_void_p, c_longlong, c_float, c_void_p],
+        "bn_rmsnorm_mean": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
+    },
+    "qk_norm": {
+        "bn_qk_norm_store": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    },
+    "state_mixers": {
+        "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
+                           c_int, c_int, c_void_p],
+        "bn_wkv_supports": [c_int, c_int],
+        "bn_wkv_scan": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                        c_int, c_void_p],
+        "bn_head_norm_gate": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+        "bn_mingru_scan": [c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int,
+                           c_void_p, c_void_p, c_int, c_void_p],
     },
     "rope_kv": {
         "bn_v_transposed_write": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
@@ -57,7 +77,7 @@ _SIGNATURES = {
         "bn_attn_rows_key_tile": [c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                         c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p],
+                         c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
     },
     "attn_mfma": {
         "bn_attn_mfma_supports": [c_int],
@@ -900,11 +920,15 @@ def _page_layout(dtype, hs: int, v_transposed, blocked) -> str:
 _LAYOUT_CODES = {"rows": 0, "transposed": 1, "blocked": 2}       # BN_KV_* of csrc/rope_kv.hip; + 4: values by page tiles
 
 
-def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None, blocked=None) -> str:
-    """Checks both page tensors against the layout that the caller names (_page_layout) and returns it.  The kernels here
-    want values as wide as keys.  Blocked pages have the shapes of pages with transposed values."""
+def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None, blocked=None, vd: int = 0) -> str:
+    """Checks both page tensors against the layout that the caller names (_page_layout) and returns it.  vd: the width
+    of a value head (0: the keys'; the vector attention kernel and qk_norm_store take another, the rest want values as
+    wide as keys).  Blocked pages have the shapes of pages with transposed values."""
+    vd = vd or hs
     layout = _page_layout(dtype, hs, v_transposed, blocked)
-    v_shape = (Hkv, PAGE, hs) if layout == "rows" else (Hkv, hs, PAGE)
+    if layout == "blocked" and vd != hs:
+        raise KernelError("blocked pages hold values as wide as keys")
+    v_shape = (Hkv, PAGE, vd) if layout == "rows" else (Hkv, vd, PAGE)
     for t, nm, shape in ((k_pages, "k_pages", (Hkv, PAGE, hs)), (v_pages, "v_pages", v_shape)):
         _dev(t, nm, dtype, 4)
         if tuple(t.shape[1:]) != shape or not t.is_contiguous():
@@ -1117,7 +1141,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
               force_vector: bool = False, fused_rotate=None, fused_write: bool = False, by_length=None,
-              max_len_dev=None, v_transposed=None, row_scale: Optional["DeferredNorm"] = None, blocked=None) -> None:
+              max_len_dev=None, v_transposed=None, row_scale: Optional["DeferredNorm"] = None, blocked=None,
+              v_dim: int = 0, distance_bias=None, sink: bool = False) -> None:
     """Causal attention of the (rotated) Q heads in qkv over the paged cache.
 
     Prompt form: `tiles` [n, 4] int32 = (sequence, first token row, tokens (<= qt), position of
@@ -1141,16 +1166,34 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     v_transposed, blocked: the layout of the pages (neither: kernel_v_layout of qkv's type and hs).
     row_scale (decode form on the matrix cores with fused_rotate): a DeferredNorm whose factor the rows of qkv still
     lack (qkv is the product of its bf16 copy with the stacked weights); the kernel multiplies q and the new key and
-    value of every row by it."""
+    value of every row by it.
+    What only the vector kernel does (pages that are not blocked): v_dim, value heads of another width than the keys'
+    (out is then [T, H * v_dim]); distance_bias = (a, b), two float32 tensors [H]: a[h] * ln(1 + b[h] * (i - j)) is taken
+    off the score of query position i and key position j; sink: the softmax has one more term of score 0 without a
+    value, i.e. 1 is added to its denominator."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
-    layout = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed, blocked)
+    vd = int(v_dim) or hs
+    layout = _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, v_transposed, blocked, vd)
     vt = layout != "rows"
     _dev(block_table, "block_table", torch.int32, 2)
     T = qkv.shape[0]
-    if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * hs) or not out.is_contiguous():
-        raise KernelError(f"attention: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} do not fit H={H} hs={hs}")
+    if H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * vd) or not out.is_contiguous():
+        raise KernelError(f"attention: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} do not fit H={H} hs={hs} v_dim={vd}")
+    if vd % 2 or vd < 2 or vd > MAX_HEAD_DIM:
+        raise KernelError(f"attention: value width {vd} is not supported (even, at most {MAX_HEAD_DIM})")
+    extras = vd != hs or distance_bias is not None or sink
+    if extras and layout == "blocked":
+        raise KernelError("attention: another value width, a distance bias and a sink are the vector kernel's, which reads "
+                          "pages with a row per position or transposed values")
+    da = db = None
+    if distance_bias is not None:
+        da, db = distance_bias
+        for t, nm in ((da, "distance_bias[0]"), (db, "distance_bias[1]")):
+            _dev(t, nm, torch.float32, 1)
+            if t.numel() != H or not t.is_contiguous():
+                raise KernelError(f"attention: {nm} must hold one float32 per head")
     if hs % 2 or hs < 2 or hs > MAX_HEAD_DIM:
         raise KernelError(f"attention: head size {hs} is not supported (even, at most {MAX_HEAD_DIM})")
     if not block_table.is_contiguous():
@@ -1195,7 +1238,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
                               f"{block_table.shape[1]} pages of the block table")
         if n_splits > (1024 if fold else 64):
             raise KernelError("attention: at most 64 splits (1,024 runs of a float32 cache)")
-        part_o = torch.empty((T * H * n_splits, hs), dtype=torch.float32, device=qkv.device)
+        part_o = torch.empty((T * H * n_splits, vd), dtype=torch.float32, device=qkv.device)
         part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
     po = part_o.data_ptr() if part_o is not None else None
     pm = part_ml.data_ptr() if part_ml is not None else None
@@ -1244,7 +1287,269 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
-        po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, int(fold), _stream()), "attention")
+        po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, int(fold), vd,
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), _stream()),
+        "attention")
+
+
+
+# --------------------------------------------------------------------------------------
+# attention without a rotation: head norms, query temperature, cache write
+# --------------------------------------------------------------------------------------
+
+def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *, v_dim: int = 0,
+                  q_weight=None, k_weight=None, eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 0,
+                  seq_index=None, block_table=None, k_pages=None, v_pages=None) -> None:
+    """In place on qkv [T, H hs + Hkv (hs + v_dim)]: every query and key head under an RMSNorm of its own (weights
+    [hs] float32, shared by the heads; both or neither), the queries times 1 + temp_coef ln(floor((p + 1) / temp_every)
+    + 1) at position p (temp_every 0: no temperature); the normed keys and the values go into the pages (a row per
+    position) when pages are given.  Rows with position < 0 are left alone."""
+    require_gpu()
+    _dev(qkv, "qkv", dims=2)
+    _dev(positions, "positions", torch.int32, 1)
+    vd = int(v_dim) or hs
+    T = qkv.shape[0]
+    if positions.numel() != T or qkv.shape[1] < H * hs + Hkv * (hs + vd) or (q_weight is None) != (k_weight is None):
+        raise KernelError(f"qk_norm_store: qkv {tuple(qkv.shape)} does not fit H={H} Hkv={Hkv} hs={hs} v_dim={vd}")
+    for w, nm in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+        if w is not None:
+            _dev(w, nm, torch.float32, 1)
+            if w.numel() != hs or not w.is_contiguous():
+                raise KernelError(f"qk_norm_store: {nm} must hold {hs} float32 values")
+    if k_pages is not None:
+        _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, False, False, vd)
+        _dev(seq_index, "seq_index", torch.int32, 1)
+        _dev(block_table, "block_table", torch.int32, 2)
+        if seq_index.numel() != T or not block_table.is_contiguous():
+            raise KernelError("qk_norm_store: one seq_index entry per row and a contiguous block table")
+    if T == 0:
+        return
+    _check(_fn("qk_norm", "bn_qk_norm_store")(
+        _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), positions.data_ptr(),
+        seq_index.data_ptr() if k_pages is not None else None, block_table.data_ptr() if k_pages is not None else None,
+        block_table.shape[1] if k_pages is not None else 0, k_pages.data_ptr() if k_pages is not None else None,
+        v_pages.data_ptr() if k_pages is not None else None, q_weight.data_ptr() if q_weight is not None else None,
+        k_weight.data_ptr() if k_weight is not None else None, T, H, Hkv, hs, vd, float(eps), float(temp_coef),
+        int(temp_every), _stream()), "qk_norm_store")
+
+
+# --------------------------------------------------------------------------------------
+# row-wise kernels of other architectures' parts
+# --------------------------------------------------------------------------------------
+
+UNARY_ACTIVATIONS = {n: _build.header_constant("BN_UNARY_" + n.upper()) for n in
+                     ("gelu_erf", "gelu_tanh", "silu", "relu2", "tanh", "sigmoid")}
+
+
+def unary_act(x: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """activation(x) element by element (float32 arithmetic); one of UNARY_ACTIVATIONS.  out: where to (x itself will do)."""
+    require_gpu()
+    _dev(x, "x")
+    if activation not in UNARY_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
+    if out is None:
+        out = torch.empty_like(x)
+    if not x.is_contiguous() or not out.is_contiguous() or out.shape != x.shape or out.dtype != x.dtype:
+        raise KernelError("unary_act: x and out must be contiguous and alike")
+    if x.numel():
+        _check(_fn("elementwise", "bn_unary_act_apply")(_code(x.dtype), out.data_ptr(), x.data_ptr(), x.numel(),
+                                                        UNARY_ACTIVATIONS[activation], _stream()), "unary_act")
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> None:
+    """In place: float32 x times a constant (an architecture's multiplier of its logits)."""
+    require_gpu()
+    _dev(x, "x", torch.float32)
+    if not x.is_contiguous():
+        raise KernelError("scale_: a contiguous float32 tensor")
+    if x.numel():
+        _check(_fn("elementwise", "bn_scale")(x.data_ptr(), x.numel(), float(factor), _stream()), "scale")
+
+
+def sinusoid_frequencies(dim: int, base: float) -> torch.Tensor:
+    """base^(-2i/dim) for i < ceil(dim / 2), formed in double and rounded to float32 once."""
+    i = torch.arange((dim + 1) // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dim).to(torch.float32)
+
+
+def embed_gather_sinusoid(table: torch.Tensor, tokens: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor,
+                          scale: float = 1.0) -> torch.Tensor:
+    """embed_gather plus a sinusoidal position vector: entry 2i gets sin(p freq[i]), entry 2i + 1 cos(p freq[i])."""
+    require_gpu()
+    _dev(table, "table", dims=2)
+    _dev(tokens, "tokens", torch.int32, 1)
+    _dev(positions, "positions", torch.int32, 1)
+    _dev(freq, "freq", torch.float32, 1)
+    n, dim = tokens.numel(), table.shape[1]
+    if (not table.is_contiguous() or not tokens.is_contiguous() or not positions.is_contiguous() or positions.numel() != n
+            or freq.numel() != (dim + 1) // 2 or not freq.is_contiguous()):
+        raise KernelError("embed_gather_sinusoid: contiguous inputs, a position per token and ceil(dim / 2) frequencies")
+    x = torch.empty((n, dim), dtype=torch.float32, device=table.device)
+    if n:
+        _check(_fn("elementwise", "bn_embed_gather_sinusoid")(
+            _code(table.dtype), x.data_ptr(), table.data_ptr(), tokens.data_ptr(), positions.data_ptr(), freq.data_ptr(),
+            n, dim, table.shape[0], float(scale), _stream()), "embed_gather_sinusoid")
+    return x
+
+
+def rmsnorm_mean(a: torch.Tensor, wa: torch.Tensor, b: Optional[torch.Tensor], wb: Optional[torch.Tensor],
+                 eps: float) -> torch.Tensor:
+    """The mean of two branches [T, D], each under an RMSNorm of its own (float32 weights [D]); b None: a alone."""
+    require_gpu()
+    _dev(a, "a", dims=2)
+    _dev(wa, "wa", torch.float32, 1)
+    T, D = a.shape
+    if not a.is_contiguous() or wa.numel() != D or not wa.is_contiguous():
+        raise KernelError("rmsnorm_mean: a contiguous [T, D] and D weights")
+    if b is not None:
+        _dev(b, "b", a.dtype, 2)
+        _dev(wb, "wb", torch.float32, 1)
+        if b.shape != a.shape or not b.is_contiguous() or wb.numel() != D or not wb.is_contiguous():
+            raise KernelError("rmsnorm_mean: the branches must be alike")
+    out = torch.empty_like(a)
+    if T:
+        _check(_fn("elementwise", "bn_rmsnorm_mean")(_code(a.dtype), out.data_ptr(), a.data_ptr(),
+                                                     b.data_ptr() if b is not None else None, wa.data_ptr(),
+                                                     wb.data_ptr() if b is not None else None, T, D, float(eps), _stream()),
+               "rmsnorm_mean")
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# mixers with a state of fixed size (csrc/state_mixers.hip)
+# --------------------------------------------------------------------------------------
+
+SEQUENCE_TILE = 1 << 30          # StepContext.tiles(SEQUENCE_TILE): one tile a sequence, for kernels that walk a sequence's tokens
+WKV_MAX_DIM = _build.header_constant("WKV_MAX_DIM", "state_mixers.hip")
+
+
+def _seq_args(tiles, seq_lens, what: str):
+    """(tiles pointer, number of tiles, seq_lens pointer): a prompt step names its sequences by tiles [n, 4], a decode
+    step by seq_lens [B] (row b = sequence b's one token)."""
+    if tiles is not None:
+        _dev(tiles, "tiles", torch.int32, 2)
+        if tiles.shape[1] != 4 or not tiles.is_contiguous():
+            raise KernelError(f"{what}: tiles must be contiguous [n, 4]")
+        return tiles.data_ptr(), tiles.shape[0], None
+    _dev(seq_lens, "seq_lens", torch.int32, 1)
+    if not seq_lens.is_contiguous():
+        raise KernelError(f"{what}: seq_lens must be contiguous")
+    return None, seq_lens.numel(), seq_lens.data_ptr()
+
+
+def _state_rows(state: torch.Tensor, need: int, what: str) -> int:
+    _dev(state, "state", torch.float32, 2)
+    if state.stride(1) != 1 or state.shape[1] < need:
+        raise KernelError(f"{what}: the state must be float32 [slots, >= {need}] with contiguous rows, got {tuple(state.shape)}")
+    return state.stride(0)
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, positions, seq_index, slot_ids) -> torch.Tensor:
+    """[n_mix, T, D]: h[t] + (h[t-1] - h[t]) * mu[s] for every mix s; the token before a step's first is read from the
+    first D values of the sequence's state row (state: [slots, >= D], a view that starts at those values), and is 0 at
+    position 0.  Reads the state only."""
+    require_gpu()
+    _dev(h, "h", dims=2)
+    _dev(mu, "mu", torch.float32, 2)
+    T, D = h.shape
+    if not h.is_contiguous() or mu.shape[1] != D or not mu.is_contiguous():
+        raise KernelError("token_shift: h contiguous [T, D], mu contiguous [n_mix, D]")
+    stride = _state_rows(state, D, "token_shift")
+    for t, nm, n in ((positions, "positions", T), (seq_index, "seq_index", T)):
+        _dev(t, nm, torch.int32, 1)
+        if t.numel() != n or not t.is_contiguous():
+            raise KernelError(f"token_shift: {nm} has one entry per row")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    out = torch.empty((mu.shape[0], T, D), dtype=h.dtype, device=h.device)
+    if T:
+        _check(_fn("state_mixers", "bn_token_shift")(_code(h.dtype), out.data_ptr(), h.data_ptr(), mu.data_ptr(), state.data_ptr(),
+                                                     stride, positions.data_ptr(), seq_index.data_ptr(),
+                                                     slot_ids.data_ptr(), T, D, mu.shape[0], _stream()), "token_shift")
+    return out
+
+
+def wkv_supported(dk: int, dv: int) -> bool:
+    return 1 <= dk <= WKV_MAX_DIM and 1 <= dv <= WKV_MAX_DIM
+
+
+def wkv_scan(r, k, v, d, w0, u, h, state, slot_ids, H: int, dk: int, dv: int, *, tiles=None, seq_lens=None) -> torch.Tensor:
+    """The wkv recurrence over every sequence of a step; float32 [T, H dv].  r, k, d: [T, H dk] (rows contiguous, any row
+    stride), v: [T, H dv], in the activations' type; w0, u: float32 [H dk] (the decay's offset, the current token's
+    bonus); h [T, D]: the mixer's input.  state [slots, >= H dk dv + D] float32: S per head as [dk, dv], then the last
+    h, both updated in place.  Per head, in float32:
+        w_t = exp(-exp(d_t + w0));  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T."""
+    require_gpu()
+    _dev(h, "h", dims=2)
+    T, D = h.shape
+    if not wkv_supported(dk, dv):
+        raise KernelError(f"wkv_scan: head sizes up to {WKV_MAX_DIM}, got {dk} x {dv}")
+    for t, nm, n in ((r, "r", H * dk), (k, "k", H * dk), (v, "v", H * dv), (d, "d", H * dk)):
+        _dev(t, nm, h.dtype, 2)
+        if t.shape != (T, n):
+            raise KernelError(f"wkv_scan: {nm} must be [{T}, {n}], got {tuple(t.shape)}")
+    for t, nm in ((w0, "w0"), (u, "u")):
+        _dev(t, nm, torch.float32, 1)
+        if t.numel() != H * dk or not t.is_contiguous():
+            raise KernelError(f"wkv_scan: {nm} must hold {H * dk} float32 values")
+    if not h.is_contiguous():
+        raise KernelError("wkv_scan: h must be contiguous")
+    stride = _state_rows(state, H * dk * dv + D, "wkv_scan")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_tiles, sl = _seq_args(tiles, seq_lens, "wkv_scan")
+    o = torch.empty((T, H * dv), dtype=torch.float32, device=h.device)
+    if T and n_tiles:
+        _check(_fn("state_mixers", "bn_wkv_scan")(
+            _code(h.dtype), r.data_ptr(), _rows(r, "r"), k.data_ptr(), _rows(k, "k"), v.data_ptr(), _rows(v, "v"),
+            d.data_ptr(), _rows(d, "d"), w0.data_ptr(), u.data_ptr(), o.data_ptr(), h.data_ptr(), state.data_ptr(), stride,
+            tl, n_tiles, sl, slot_ids.data_ptr(), H, dk, dv, D, _stream()), "wkv_scan")
+    return o
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, H: int, dv: int, eps: float) -> torch.Tensor:
+    """o [T, H dv] float32, each head divided by its root mean square (eps inside the root), times weight [H dv]
+    (float32), times silu(gate) (gate [T, H dv] in the activations' type, which is the result's)."""
+    require_gpu()
+    _dev(o, "o", torch.float32, 2)
+    _dev(gate, "gate", dims=2)
+    _dev(weight, "weight", torch.float32, 1)
+    T = o.shape[0]
+    if o.shape[1] != H * dv or not o.is_contiguous() or gate.shape != o.shape or weight.numel() != H * dv or not weight.is_contiguous():
+        raise KernelError("head_norm_gate: o and gate [T, H dv], weight [H dv]")
+    y = torch.empty((T, H * dv), dtype=gate.dtype, device=o.device)
+    if T:
+        _check(_fn("state_mixers", "bn_head_norm_gate")(_code(gate.dtype), y.data_ptr(), o.data_ptr(), gate.data_ptr(),
+                                                        _rows(gate, "gate"), weight.data_ptr(), T, H, dv, float(eps), _stream()),
+               "head_norm_gate")
+    return y
+
+
+def mingru_scan(zxg: torch.Tensor, bias_z, bias_x, state: torch.Tensor, slot_ids, W: int, *, tiles=None,
+                seq_lens=None) -> torch.Tensor:
+    """The min-GRU recurrence over every sequence of a step.  zxg [T, 3 W]: the projections of the update gate, the
+    candidate and the output gate side by side, without biases (bias_z, bias_x: float32 [W] or None).  state
+    [slots, >= W] float32, updated in place.  Per channel, in float32: z = sigmoid(a + bias_z); c = b + bias_x;
+    cand = c + 1/2 where c >= 0, sigmoid(c) below; S <- (1 - z) S + z cand; result S * silu(g), [T, W]."""
+    require_gpu()
+    _dev(zxg, "zxg", dims=2)
+    T = zxg.shape[0]
+    if zxg.shape[1] != 3 * W:
+        raise KernelError(f"mingru_scan: zxg must be [T, {3 * W}], got {tuple(zxg.shape)}")
+    for t, nm in ((bias_z, "bias_z"), (bias_x, "bias_x")):
+        if t is not None:
+            _dev(t, nm, torch.float32, 1)
+            if t.numel() != W or not t.is_contiguous():
+                raise KernelError(f"mingru_scan: {nm} must hold {W} float32 values")
+    stride = _state_rows(state, W, "mingru_scan")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_tiles, sl = _seq_args(tiles, seq_lens, "mingru_scan")
+    y = torch.empty((T, W), dtype=zxg.dtype, device=zxg.device)
+    if T and n_tiles:
+        _check(_fn("state_mixers", "bn_mingru_scan")(
+            _code(zxg.dtype), y.data_ptr(), zxg.data_ptr(), _rows(zxg, "zxg"),
+            bias_z.data_ptr() if bias_z is not None else None, bias_x.data_ptr() if bias_x is not None else None,
+            state.data_ptr(), stride, tl, n_tiles, sl, slot_ids.data_ptr(), W, _stream()), "mingru_scan")
+    return y
 
 
 # --------------------------------------------------------------------------------------

@@ -10,6 +10,16 @@ to the last `window` positions.
 The three projections are stored stacked ([Wq; Wk; Wv], as the reference's GPU upload
 stacks them, include/backend_model.h:21-22) so that one product computes them.
 A schedule entry that reads another entry's cache computes Q only.
+
+What other architectures put into the same mixer, each a parameter that is off by default; any of them takes the
+mixer to the vector kernel over pages with a row per position, in both types, and needs position "none":
+  v_head_dim     value heads of another width than the query/key heads
+  qk_norm_eps    an RMSNorm over every query and every key head before they meet (tensors q_norm, k_norm [head_dim],
+                 shared by the heads, plain weights)
+  q_temp_coef, q_temp_every   the query at position p times 1 + coef * ln(floor((p + 1) / every) + 1)
+  distance_bias  tensors dist_a, dist_b [heads]: dist_a[h] * ln(1 + dist_b[h] * (i - j)) is taken off the score of
+                 query i and key j
+  sink           the softmax has one more term of score 0 and no value: p_j = exp(s_j) / (1 + sum exp(s))
 """
 from __future__ import annotations
 
@@ -30,7 +40,9 @@ class Attention(Part):
     gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
 
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
-                 position: PartSpec, window: int = 0, bias: bool = False):
+                 position: PartSpec, window: int = 0, bias: bool = False, v_head_dim: int = 0,
+                 qk_norm_eps: float | None = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
+                 distance_bias: bool = False, sink: bool = False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
         if head_dim % 2 or head_dim < 2 or head_dim > ops.MAX_HEAD_DIM:
@@ -40,6 +52,20 @@ class Attention(Part):
         self.scale, self.window, self.has_bias = float(scale), int(window), bool(bias)
         self.position = POSITION_ENCODINGS.build(position)
         self.qkv, self.o = Linear(), Linear()
+        self.vd = int(v_head_dim) or self.hs
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.q_temp_coef, self.q_temp_every = float(q_temp_coef), int(q_temp_every)
+        self.distance_bias, self.sink = bool(distance_bias), bool(sink)
+        self.general = (self.vd != self.hs or self.qk_norm_eps is not None or self.q_temp_every > 0
+                        or self.distance_bias or self.sink)
+        if self.general:
+            if self.vd % 2 or self.vd < 2 or self.vd > ops.MAX_HEAD_DIM:
+                raise ValueError(f"attention: v_head_dim {self.vd} is not supported by the kernels (even, at most {ops.MAX_HEAD_DIM})")
+            if self.position.rope_dims or self.has_bias:
+                raise ValueError("attention: head norms, a query temperature, a distance bias, a sink or values of another "
+                                 "width come without a rotation and without projection biases")
+            self.takes_deferred_norm = self.gives_lazy_delta = False
+        self.q_norm = self.k_norm = self.dist_a = self.dist_b = None
 
     @property
     def q_dim(self):
@@ -51,7 +77,11 @@ class Attention(Part):
 
     def tensors(self):
         t = {"wq": ParamSpec((self.q_dim, self.hidden)), "wk": ParamSpec((self.kv_dim, self.hidden)),
-             "wv": ParamSpec((self.kv_dim, self.hidden)), "wo": ParamSpec((self.hidden, self.q_dim))}
+             "wv": ParamSpec((self.Hkv * self.vd, self.hidden)), "wo": ParamSpec((self.hidden, self.H * self.vd))}
+        if self.qk_norm_eps is not None:
+            t.update({"q_norm": ParamSpec((self.hs,), "ones"), "k_norm": ParamSpec((self.hs,), "ones")})
+        if self.distance_bias:
+            t.update({"dist_a": ParamSpec((self.H,), "normal"), "dist_b": ParamSpec((self.H,), "ones")})
         if self.has_bias:
             t.update({"bq": ParamSpec((self.q_dim,), "normal"), "bk": ParamSpec((self.kv_dim,), "normal"),
                       "bv": ParamSpec((self.kv_dim,), "normal"), "bo": ParamSpec((self.hidden,), "normal")})
@@ -59,18 +89,24 @@ class Attention(Part):
 
     def load(self, tensors, device, dtype):
         # stacked on the device: the host holds no copy beside the file's own bytes
-        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wq", "wk", "wv")], dim=0)
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wq", "wk", "wv")], dim=0).contiguous()
         b = None
         if self.has_bias:
             b = torch.cat([upload(tensors[n], device, torch.float32) for n in ("bq", "bk", "bv")])
         self.qkv.load(w, b, device, dtype)
         self.o.load(tensors["wo"], tensors.get("bo") if self.has_bias else None, device, dtype)
         self.position.prepare(device)
+        if self.qk_norm_eps is not None:
+            self.q_norm, self.k_norm = (upload(tensors[n], device, torch.float32) for n in ("q_norm", "k_norm"))
+        if self.distance_bias:
+            self.dist_a, self.dist_b = (upload(tensors[n], device, torch.float32) for n in ("dist_a", "dist_b"))
 
     def linears(self):
         return [self.qkv, self.o]
 
     def cache_need(self) -> CacheNeed:
+        if self.general:                  # the vector kernel's pages, in both types
+            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_head_dim=self.vd, v_layout="rows"))
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 
     def wants_deferred_norm(self, ctx, rows: int) -> bool:
@@ -82,7 +118,40 @@ class Attention(Part):
         return bool(ctx.is_decode and fuse_ok and inv_freq is not None and not self.has_bias and ops.LIBRARY_PRODUCTS
                     and ops.can_fuse_decode(self.qkv.weight.dtype, self.H, self.Hkv, self.hs))
 
+    def _forward_general(self, h, ctx, kv):
+        """Projections, head norms and temperature with the cache write (one kernel), the vector attention kernel with
+        its distance bias and sink, the output projection."""
+        H, Hkv, hs, vd = self.H, self.Hkv, self.hs, self.vd
+        if isinstance(h, ops.DeferredNorm):
+            h = h.materialize()
+        width = H * hs + Hkv * (hs + vd)
+        if kv.writes:
+            qkv = self.qkv(h)
+        else:
+            qkv = torch.empty((h.shape[0], width), dtype=h.dtype, device=h.device)
+            qkv[:, :self.q_dim] = self.qkv(h, rows=slice(0, self.q_dim))
+        ops.qk_norm_store(qkv, ctx.positions, H, Hkv, hs, v_dim=vd, q_weight=self.q_norm, k_weight=self.k_norm,
+                          eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
+                          seq_index=ctx.seq_index if kv.writes else None, block_table=kv.block_table if kv.writes else None,
+                          k_pages=kv.k_pages if kv.writes else None, v_pages=kv.v_pages if kv.writes else None)
+        out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
+        bias = (self.dist_a, self.dist_b) if self.distance_bias else None
+        if ctx.is_decode:
+            n_splits, chunk = (1, 0) if self.window else ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
+            ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
+                          seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=False, blocked=False,
+                          v_dim=vd, distance_bias=bias, sink=self.sink)
+        else:
+            _, _, qt = ops.attention_row_shape(H, Hkv, False)
+            ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
+                          tiles=ctx.tiles(qt), qt=qt, v_transposed=False, blocked=False, v_dim=vd, distance_bias=bias,
+                          sink=self.sink)
+        return self.o(out)
+
     def forward(self, h, ctx, kv, lazy_ok: bool = False):
+        if self.general:
+            return self._forward_general(h, ctx, kv)
         H, Hkv, hs = self.H, self.Hkv, self.hs
         last = self.o.lazy if lazy_ok else self.o
         fuse_ok, inv_freq = self.position.fusable(hs)

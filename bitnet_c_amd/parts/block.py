@@ -1,7 +1,8 @@
 """Arrangement of the parts of one layer.
 
 "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) -- the order of the reference's layer
-(src/transformer/cpu.c:536-939 and :1247-1303): norm, mixer, add, norm, feed-forward, add."""
+(src/transformer/cpu.c:536-939 and :1247-1303): norm, mixer, add, norm, feed-forward, add.
+A layer without a feed-forward (ffn None; ffn_norm None with it) is the first half alone."""
 from __future__ import annotations
 
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, PartSpec
@@ -9,18 +10,21 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, PartSpec
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Part):
-    def __init__(self, mixer: PartSpec, ffn: PartSpec, mixer_norm: PartSpec, ffn_norm: PartSpec):
+    def __init__(self, mixer: PartSpec, ffn: PartSpec | None, mixer_norm: PartSpec, ffn_norm: PartSpec | None = None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("prenorm block: a feed-forward and its norm come together or not at all")
         self.mixer = MIXERS.build(mixer)
-        self.ffn = FEED_FORWARDS.build(ffn)
+        self.ffn = FEED_FORWARDS.build(ffn) if ffn is not None else None
         self.mixer_norm = NORMS.build(mixer_norm)
-        self.ffn_norm = NORMS.build(ffn_norm)
+        self.ffn_norm = NORMS.build(ffn_norm) if ffn_norm is not None else None
 
     @property
     def prompt_capturable(self) -> bool:
         return all(getattr(c, "prompt_capturable", False) for c in self.children().values())
 
     def children(self):
-        return {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}
+        c = {"mixer": self.mixer, "ffn": self.ffn, "mixer_norm": self.mixer_norm, "ffn_norm": self.ffn_norm}
+        return {k: v for k, v in c.items() if v is not None}
 
     def linears(self):
         return [l for part in self.children().values() for l in getattr(part, "linears", list)()]
@@ -48,6 +52,10 @@ class PreNormBlock(Part):
             stream.add(self.mixer.forward(h, ctx, kv))
         if tap is not None:
             tap("ffn_in", ctx.entry, stream, ctx)
+        if self.ffn is None:
+            if tap is not None:
+                tap("layer_out", ctx.entry, stream, ctx)
+            return
         h = stream.normed(self.ffn_norm, ctx.act_dtype, consumer=self.ffn, ctx=ctx)
         if getattr(self.ffn, "gives_lazy_delta", False):
             stream.add(self.ffn.forward(h, ctx, lazy_ok=True))

@@ -14,6 +14,36 @@ from .base import FEED_FORWARDS, ParamSpec, Part
 from .linear import Linear, upload
 
 
+@FEED_FORWARDS.register("dense")
+class DenseFFN(Part):
+    """A feed-forward without a gate: down(act(up(x))).  act is one of ops.UNARY_ACTIVATIONS ("gelu_erf": the exact
+    gelu, 0.5 z (1 + erf(z / sqrt 2)); the others as the gated unit's)."""
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+    takes_deferred_norm = True      # forward accepts an ops.DeferredNorm for h (the first product applies the norm)
+    gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "gelu_erf"):
+        if activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"feed-forward: unknown activation {activation!r}; known: {sorted(ops.UNARY_ACTIVATIONS)}")
+        self.hidden, self.F, self.activation = int(hidden), int(intermediate), activation
+        self.up, self.down = Linear(), Linear()
+
+    def tensors(self):
+        return {"w_up": ParamSpec((self.F, self.hidden)), "w_down": ParamSpec((self.hidden, self.F))}
+
+    def load(self, tensors, device, dtype):
+        self.up.load(tensors["w_up"], None, device, dtype)
+        self.down.load(tensors["w_down"], None, device, dtype)
+
+    def linears(self):
+        return [self.up, self.down]
+
+    def forward(self, h, ctx, lazy_ok: bool = False):
+        a = self.up(h)
+        ops.unary_act(a, self.activation, out=a)
+        return self.down.lazy(a) if lazy_ok else self.down(a)
+
+
 @FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(Part):

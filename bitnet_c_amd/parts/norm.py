@@ -1,6 +1,8 @@
 """RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * w, eps inside the root
 (src/transformer/rmsnorm_scalar.c:4-13).  Computed in float32 whatever the activation
-type; the weight is kept in float32."""
+type; the weight is kept in float32.  `scalar`: the model folder holds one number for all
+coordinates (a tensor without dimensions); it is spread over the coordinates at load, and
+every kernel that takes this norm, folded into a product or not, sees a weight vector."""
 from __future__ import annotations
 
 import torch
@@ -16,15 +18,16 @@ class RMSNorm(Part):
     deferrable = True        # a product may fold this norm around itself (weight and eps are all it needs)
     takes_partial_sums = True    # apply() accepts ops.PartialSums as the delta
 
-    def __init__(self, dim: int, eps: float):
-        self.dim, self.eps = int(dim), float(eps)
+    def __init__(self, dim: int, eps: float, scalar: bool = False):
+        self.dim, self.eps, self.scalar = int(dim), float(eps), bool(scalar)
         self.weight = None
 
     def tensors(self):
-        return {"weight": ParamSpec((self.dim,), init="ones")}
+        return {"weight": ParamSpec(() if self.scalar else (self.dim,), init="ones")}
 
     def load(self, tensors, device, dtype):
-        self.weight = upload(tensors["weight"], device, torch.float32)
+        w = upload(tensors["weight"], device, torch.float32)
+        self.weight = w.reshape(1).expand(self.dim).contiguous() if self.scalar else w
 
     def apply(self, x, delta, out_dtype, rows=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, out_dtype, rows)

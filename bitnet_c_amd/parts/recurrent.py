@@ -1,0 +1,123 @@
+"""Mixers that carry a state of fixed size per sequence instead of keys and values.  The state lives in the cache's
+state area (float32, a row per sequence slot, zero when a slot is handed out) and is addressed through the step's
+device-side slot ids alone, so decode steps and prompt steps of models with these mixers are captured like any other.
+Whatever enters a recurrence is float32 (decays, gates, exponentials, the state); the projections run in the
+activations' type.  The kernels are csrc/state_mixers.hip.
+
+"wkv": time mixing with a matrix state per head and a decay that depends on the token.  With h' the previous token's
+input (zero before the first token; the last h of a step is part of the state):
+    x_s = h + (h' - h) * mu_s                     for s in r, k, v, g, w  (five mixes of the same two rows)
+    r, k, v = W_r x_r, W_k x_k, W_v x_v           heads x head_dim each;  gate = silu(W_g x_g)
+    w = exp(-exp(W_w2 tanh(W_w1 x_w) + w0))       per head and key channel, in (0, 1)
+    o_t = (S + diag(u) k_t v_t^T)^T r_t           the bonus u counts for the current token alone
+    S  <- diag(w_t) S + k_t v_t^T
+    y = W_o (o / rms_head(o) * norm * gate)       every head divided by its own root mean square (eps inside the root)
+
+"mingru": a gated recurrence whose gates read the current token alone:
+    z = sigmoid(W_z h + b_z);  c = W_x h + b_x;  cand = c + 1/2 where c >= 0, sigmoid(c) below
+    S <- (1 - z) S + z cand   element by element;   y = W_o (S * silu(W_g h))
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import MIXERS, CacheNeed, ParamSpec, Part, StateNeed
+from .linear import Linear, upload
+
+
+def _sequences(ctx):
+    """How a kernel that walks a sequence's tokens finds them: one tile a sequence in a prompt step, the lengths in a
+    decode step (row b is sequence b's one token)."""
+    if ctx.is_decode:
+        return dict(seq_lens=ctx.seq_lens)
+    return dict(tiles=ctx.tiles(ops.SEQUENCE_TILE))
+
+
+@MIXERS.register("wkv")
+class WKV(Part):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, hidden: int, n_heads: int, head_dim: int, decay_rank: int, eps: float):
+        self.hidden, self.H, self.hs, self.rank, self.eps = int(hidden), int(n_heads), int(head_dim), int(decay_rank), float(eps)
+        if not ops.wkv_supported(self.hs, self.hs):
+            raise ValueError(f"wkv: head_dim {self.hs} is not supported by the kernel (at most {ops.WKV_MAX_DIM})")
+        self.r, self.k, self.v, self.g, self.w1, self.w2, self.o = (Linear() for _ in range(7))
+        self.mu = self.w0 = self.u = self.norm = None
+
+    @property
+    def inner(self):
+        return self.H * self.hs
+
+    def tensors(self):
+        D, A = self.hidden, self.inner
+        t = {f"mu_{s}": ParamSpec((D,), "normal") for s in self.MIXES}
+        t.update({"wr": ParamSpec((A, D)), "wk": ParamSpec((A, D)), "wv": ParamSpec((A, D)), "wg": ParamSpec((A, D)),
+                  "w1": ParamSpec((self.rank, D)), "w2": ParamSpec((A, self.rank)), "w0": ParamSpec((A,), "normal"),
+                  "u": ParamSpec((self.H, self.hs), "normal"), "norm": ParamSpec((A,), "ones"), "wo": ParamSpec((D, A))})
+        return t
+
+    def load(self, tensors, device, dtype):
+        for lin, n in ((self.r, "wr"), (self.k, "wk"), (self.v, "wv"), (self.g, "wg"), (self.w1, "w1"), (self.w2, "w2"),
+                       (self.o, "wo")):
+            lin.load(tensors[n], None, device, dtype)
+        self.mu = torch.stack([upload(tensors[f"mu_{s}"], device, torch.float32) for s in self.MIXES]).contiguous()
+        self.w0 = upload(tensors["w0"], device, torch.float32)
+        self.u = upload(tensors["u"], device, torch.float32).reshape(-1).contiguous()
+        self.norm = upload(tensors["norm"], device, torch.float32)
+
+    def linears(self):
+        return [self.r, self.k, self.v, self.g, self.o]
+
+    def cache_need(self) -> CacheNeed:
+        # per head a [head_dim, head_dim] matrix, then the last input row
+        return CacheNeed(state=StateNeed((self.inner * self.hs + self.hidden,), torch.float32, device_addressed=True))
+
+    def forward(self, h, ctx, kv):
+        H, hs = self.H, self.hs
+        state = kv.state
+        mixes = ops.token_shift(h, self.mu, state[:, self.inner * hs:], ctx.positions, ctx.seq_index, ctx.slot_ids)
+        r, k, v, g = self.r(mixes[0]), self.k(mixes[1]), self.v(mixes[2]), self.g(mixes[3])
+        low = self.w1(mixes[4])
+        ops.unary_act(low, "tanh", out=low)
+        d = self.w2(low)
+        o = ops.wkv_scan(r, k, v, d, self.w0, self.u, h, state, ctx.slot_ids, H, hs, hs, **_sequences(ctx))
+        y = ops.head_norm_gate(o, g, self.norm, H, hs, self.eps)
+        return self.o(y)
+
+
+@MIXERS.register("mingru")
+class MinGRU(Part):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+
+    def __init__(self, hidden: int, width: int, bias: bool = True):
+        self.hidden, self.W, self.has_bias = int(hidden), int(width), bool(bias)
+        self.zxg, self.o = Linear(), Linear()         # the three projections stacked: one product
+        self.bz = self.bx = None
+
+    def tensors(self):
+        D, W = self.hidden, self.W
+        t = {"wz": ParamSpec((W, D)), "wx": ParamSpec((W, D)), "wg": ParamSpec((W, D)), "wo": ParamSpec((D, W))}
+        if self.has_bias:
+            t.update({"bz": ParamSpec((W,), "normal"), "bx": ParamSpec((W,), "normal")})
+        return t
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wz", "wx", "wg")], dim=0).contiguous()
+        self.zxg.load(w, None, device, dtype)
+        self.o.load(tensors["wo"], None, device, dtype)
+        if self.has_bias:
+            self.bz, self.bx = (upload(tensors[n], device, torch.float32) for n in ("bz", "bx"))
+
+    def linears(self):
+        return [self.zxg, self.o]
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(state=StateNeed((self.W,), torch.float32, device_addressed=True))
+
+    def forward(self, h, ctx, kv):
+        zxg = self.zxg(h)
+        y = ops.mingru_scan(zxg, self.bz, self.bx, kv.state, ctx.slot_ids, self.W, **_sequences(ctx))
+        return self.o(y)

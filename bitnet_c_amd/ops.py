@@ -1284,7 +1284,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
             "attention(mfma)")
         return
     _check(_fn("attn_rows", "bn_attn_rows")(
-        _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * hs,
+        _code(qkv.dtype), qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * vd,
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
         po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, int(fold), vd,

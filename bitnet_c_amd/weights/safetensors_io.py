@@ -160,5 +160,5 @@ def write_file(path: str, tensors: Dict[str, torch.Tensor], metadata: dict | Non
         f.write(blob)
         for name in order:
             t = tensors[name].detach().cpu().contiguous()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")     # reshape: a tensor without dimensions too
     os.replace(tmp, path)

@@ -168,6 +168,106 @@ KERNEL_WORKLOADS = {"skinny": _kernel_skinny, "gemm": _kernel_gemm, "attention_p
                     "attention_decode": _kernel_attention_decode, "mid": _kernel_mid}
 
 
+# ---- another design beside the Llama-style decoder at equal size (--design) ----------------------------------------
+# Layer sizes that resemble real models: width, feed-forward, 64-wide recurrence heads, attention heads of 128.
+DESIGN_SIZES = {
+    "2048": dict(width=2048, ff=8192, rec_heads=32, rec_dim=64, rank=64, heads=16, kv_heads=4, dim=128, right=2048,
+                 vocab=32000, layers=12),
+    "4096": dict(width=4096, ff=16384, rec_heads=64, rec_dim=64, rank=128, heads=32, kv_heads=8, dim=128, right=4096,
+                 vocab=32000, layers=9),
+}
+
+
+def _design_configs(z):
+    """(Sunusun config.json, Llama config.json) of equal width, layers, attention heads and (nearly) equal weight bytes:
+    two recurrent layers, then one parallel layer, repeated; the gated feed-forward is 2/3 as wide as the dense one."""
+    wkv = dict(type="wkv", mixer=dict(heads=z["rec_heads"], dim=z["rec_dim"], decay_rank=z["rank"]),
+               mlp=dict(kind="dense", ff=z["ff"]))
+    par = dict(type="parallel", mlp=dict(kind="dense", ff=z["ff"]), mixer=dict(
+        left=dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+                  q_temp=dict(coef=0.1, every=256)), right=dict(width=z["right"])))
+    sun = dict(architecture="Sunusun", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6), logit_scale=1.0,
+               layers=[par if i % 3 == 2 else wkv for i in range(z["layers"])])
+    llama = dict(model_type="llama", vocab_size=z["vocab"], hidden_size=z["width"],
+                 intermediate_size=(2 * z["ff"] // 3 + 255) // 256 * 256, num_hidden_layers=z["layers"],
+                 num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                 max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+    return sun, llama
+
+
+def bench_design(args) -> int:
+    import torch
+
+    import bitnet_c_amd as bn
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.config import architecture_for
+    from bitnet_c_amd.engine import DecoderModel
+    from bitnet_c_amd.sampling import SamplingParams, SequenceSampler, start_sampling
+    from bitnet_c_amd.weights import random_tensors
+
+    dev, z = "cuda:0", DESIGN_SIZES[args.design_size]
+    rnd = random.Random(args.seed)
+    batches = (1, 8, 64)
+    PREFILL, lens = args.prefill_tokens, (256, 1024)
+    out = {"design": args.design, "size": args.design_size, "sizes": z, "dtype": "bf16", "steps": args.steps, "warmup": args.warmup,
+           "prefill_tokens": PREFILL, "decode_prompt_lens": list(lens), "data": "synthetic: random N(0,0.02) weights, uniform token ids"}
+    for name, raw in zip((args.design, "llama"), _design_configs(z)):
+        arch = architecture_for(raw)
+        cfg = arch.config_cls.from_dict(raw)
+        plan = arch.build_plan(cfg)
+        model = DecoderModel(plan, torch.bfloat16, dev)
+        model.load(random_tensors(plan.expected_tensors(), args.seed, torch.bfloat16, device=dev))
+        per_seq = ((lens[1] + args.steps + args.warmup + 64 + 63) // 64) * 64
+        engine = bn.Engine(model, max_tokens=max(batches[-1] * per_seq, PREFILL + 64), max_slots=batches[-1] + 1)
+        vocab = plan.vocab_size
+        rec = {"weight_gb": round(model.weight_bytes() / 1e9, 3)}
+
+        def prefill_once():
+            s = engine.new_sequence()
+            toks = [rnd.randrange(vocab) for _ in range(PREFILL)]
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            ops.argmax(engine.step([bn.StepEntry(s, toks, [PREFILL - 1])])).cpu()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            engine.release(s)
+            return dt
+
+        if args.only != "decode":
+            prefill_once()
+            prefill_once()
+            ms = sorted(prefill_once() for _ in range(5))[2] * 1e3
+            rec["prefill_ms"], rec["prefill_tok_s"] = round(ms, 3), round(PREFILL / ms * 1e3, 1)
+        for b in batches if args.only != "prefill" else ():
+            slots = [engine.new_sequence() for _ in range(b)]
+            last = []
+            for s in slots:
+                n = rnd.randint(*lens)
+                last += ops.argmax(engine.step([bn.StepEntry(s, [rnd.randrange(vocab) for _ in range(n)], [n - 1])])).cpu().tolist()
+            greedy = [SequenceSampler(SamplingParams())] * b
+            entries = [bn.StepEntry(s, [0], [0]) for s in slots]
+            engine.prepare_decode(b)
+            lg = engine.step([bn.StepEntry(s, [t], [0]) for s, t in zip(slots, last)])
+            for i in range(args.warmup + args.steps):
+                if i == args.warmup:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                pending = start_sampling(lg, greedy)
+                lg = engine.step(entries, device_tokens=pending.device_tokens)
+                pending.tokens()
+            torch.cuda.synchronize()
+            step = (time.perf_counter() - t0) / args.steps
+            for s in slots:
+                engine.release(s)
+            rec[f"decode_b{b}_ms"], rec[f"decode_b{b}_tok_s"] = round(step * 1e3, 4), round(b / step, 1)
+        print(f"[bench] {name}: {rec}", file=sys.stderr, flush=True)
+        out[name] = rec
+        del engine, model
+        torch.cuda.empty_cache()
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,7 +286,16 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=0, help="longest sequence (default: the shape's)")
     ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the measured prompt step")
+    ap.add_argument("--design", choices=["sunusun"], default=None,
+                    help="instead of the benchmark: prefill and decode of this design beside the Llama-style decoder of equal "
+                         "width, heads, layers and weight bytes, at the sizes of --design-size (random weights; one JSON line)")
+    ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="2048")
     args = ap.parse_args()
+    if args.design:
+        if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+            print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+            return 2
+        return bench_design(args)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2

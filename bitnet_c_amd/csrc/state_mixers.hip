@@ -68,12 +68,17 @@ extern "C" int bn_token_shift(int dtype, void* out, const void* h, const float* 
 
 // ---- the wkv recurrence -----------------------------------------------------------------------------------------------
 // A workgroup owns (sequence, head, a block of CB value columns).  Column j of a head's state S[dk, dv] depends on no
-// other column, so the columns are spread over threads and workgroups freely; the dk rows of a column are spread over
-// P threads (P a power of two <= 64, neighbouring lanes), each holding up to WKV_KR rows in registers, row i = p + P ii.
-// The tokens of a sequence come in chunks of TC: r, k, the decay and the block's v are staged in shared memory once a
-// chunk (rows beyond dk zero, which leaves the unused registers zero), then the chunk's tokens run without a barrier.
+// other column, so the columns are spread over threads and workgroups freely (the host picks CB so that a launch fills
+// the chip); the dk rows of a column are spread over P threads (P a power of two <= 16, neighbouring lanes), each holding
+// WKV_KR consecutive rows in registers, rows p WKV_KR .. p WKV_KR + WKV_KR - 1.  The tokens of a sequence come in chunks
+// of TC: r, k, the decay and the block's v are staged in shared memory once a chunk (rows beyond dk zero, which leaves the
+// unused registers zero) by waves of the workgroup that do nothing else: while the walking waves run a chunk's tokens
+// without a barrier, every thread reading its rows 16 bytes at a time, the staging waves fill the other buffer with the
+// next chunk, exponentials of the decay included, so the walk never waits for memory.  A column's sum over the rows is formed in four
+// partial sums per thread and a butterfly over the P threads: an order that depends on the head size alone.
 #define WKV_KR 16
 #define WKV_MAX_DIM 256
+#define WKV_MAX_THREADS 256
 
 struct WkvArgs {
     const void* r; const void* k; const void* v; const void* d;     // [T, ld*]: head h at h * dk (v: h * dv)
@@ -85,79 +90,100 @@ struct WkvArgs {
     float* state;             // [slots, state_stride]: S as [H][dk][dv], then D values of the last h
     size_t state_stride;
     const int* tiles; const int* seq_lens; const int* slot_ids;
-    int H, dk, dv, D, P, CB, TC;
+    int H, dk, dv, D, P, CB, TC, walkers;
 };
 
 template <typename T>
-__global__ void wkv_scan_kernel(WkvArgs a) {
-    extern __shared__ float smem[];
+__global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs a) {
+    extern __shared__ __align__(16) float smem[];
     const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
     if (sr.n <= 0 || sr.pos0 < 0) return;
     const int head = blockIdx.y, cb = blockIdx.z;
-    const int P = a.P, dk = a.dk, dv = a.dv, TC = a.TC;
+    const int P = a.P, dk = a.dk, dv = a.dv, TC = a.TC, CB = a.CB;
     const int dkp = P * WKV_KR;                           // staged rows, zero beyond dk
     const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int n_walk = a.walkers;                         // the first n_walk threads walk the tokens, the rest stage them
+    const bool walker = tid < n_walk;
     const int p = tid % P, jl = tid / P;
-    const int j = cb * a.CB + jl;                         // this thread's value column
-    const bool owns = jl < a.CB && j < dv;
-    float* r_s = smem;                                    // [TC][dkp]
-    float* k_s = r_s + TC * dkp;
-    float* w_s = k_s + TC * dkp;
-    float* v_s = w_s + TC * dkp;                          // [TC][CB]
+    const int j = cb * CB + jl;                           // a walker's value column
+    const bool owns = walker && jl < CB && j < dv;
+    const int buf_floats = TC * (3 * dkp + CB);           // one staged chunk: r, k, w as [TC][dkp], then v as [TC][CB]
 
     float* S_g = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * dk * dv;
     float S[WKV_KR], ub[WKV_KR];
 #pragma unroll
     for (int ii = 0; ii < WKV_KR; ++ii) {
-        const int i = p + P * ii;
+        const int i = p * WKV_KR + ii;
         const bool in = owns && i < dk;
         S[ii] = (in && sr.pos0 > 0) ? S_g[(size_t)i * dv + j] : 0.f;
-        ub[ii] = (in) ? a.u[(size_t)head * dk + i] : 0.f;
+        ub[ii] = in ? a.u[(size_t)head * dk + i] : 0.f;
     }
 
-    for (int c0 = 0; c0 < sr.n; c0 += TC) {
-        const int nc = min(TC, sr.n - c0);
-        __syncthreads();                                  // the chunk before this one has been consumed
-        for (int idx = tid; idx < nc * dkp; idx += nthreads) {
+    // the staging threads' work: chunk c0 into buffer b
+    auto stage = [&](int c0, int b) {
+        float* r_s = smem + (size_t)b * buf_floats;
+        float* k_s = r_s + TC * dkp;
+        float* w_s = k_s + TC * dkp;
+        float* v_s = w_s + TC * dkp;
+        const int nc = min(TC, sr.n - c0), lt = tid - n_walk, nl = nthreads - n_walk;
+        for (int idx = lt; idx < nc * dkp; idx += nl) {
             const int tt = idx / dkp, i = idx - tt * dkp;
-            const size_t row = (size_t)(sr.row0 + c0 + tt);
             float rv = 0.f, kv = 0.f, wv = 0.f;
             if (i < dk) {
-                const size_t c = (size_t)head * dk + i;
+                const size_t row = (size_t)(sr.row0 + c0 + tt), c = (size_t)head * dk + i;
                 rv = to_f32(reinterpret_cast<const T*>(a.r)[row * a.ldr + c]);
                 kv = to_f32(reinterpret_cast<const T*>(a.k)[row * a.ldk + c]);
                 wv = expf(-expf(to_f32(reinterpret_cast<const T*>(a.d)[row * a.ldd + c]) + a.w0[c]));
             }
             r_s[idx] = rv; k_s[idx] = kv; w_s[idx] = wv;
         }
-        for (int idx = tid; idx < nc * a.CB; idx += nthreads) {
-            const int tt = idx / a.CB, c = idx - tt * a.CB;
-            const int col = cb * a.CB + c;
+        for (int idx = lt; idx < nc * CB; idx += nl) {
+            const int tt = idx / CB, col = cb * CB + (idx - tt * CB);
             v_s[idx] = col < dv ? to_f32(reinterpret_cast<const T*>(a.v)[(size_t)(sr.row0 + c0 + tt) * a.ldv +
                                                                           (size_t)head * dv + col]) : 0.f;
         }
-        __syncthreads();
-        if (jl < a.CB) {
+    };
+
+    if (!walker) stage(0, 0);
+    __syncthreads();
+    int b = 0;
+    for (int c0 = 0; c0 < sr.n; c0 += TC, b ^= 1) {
+        const int nc = min(TC, sr.n - c0);
+        if (!walker) {
+            if (c0 + TC < sr.n) stage(c0 + TC, b ^ 1);
+        } else if (jl < CB) {
+            const float* r_s = smem + (size_t)b * buf_floats;
+            const float* k_s = r_s + TC * dkp;
+            const float* w_s = k_s + TC * dkp;
+            const float* v_s = w_s + TC * dkp;
             for (int tt = 0; tt < nc; ++tt) {
-                const float vj = v_s[tt * a.CB + jl];
-                const float* rr = r_s + tt * dkp + p;
-                const float* kk = k_s + tt * dkp + p;
-                const float* ww = w_s + tt * dkp + p;
-                float acc = 0.f;
+                const float vj = v_s[tt * CB + jl];
+                const float4* rr = reinterpret_cast<const float4*>(r_s + tt * dkp + p * WKV_KR);
+                const float4* kk = reinterpret_cast<const float4*>(k_s + tt * dkp + p * WKV_KR);
+                const float4* ww = reinterpret_cast<const float4*>(w_s + tt * dkp + p * WKV_KR);
+                float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ii = 0; ii < WKV_KR; ++ii) {
-                    const float kv = kk[P * ii] * vj;
-                    acc = fmaf(rr[P * ii], fmaf(ub[ii], kv, S[ii]), acc);
-                    S[ii] = fmaf(ww[P * ii], S[ii], kv);
+                for (int q4 = 0; q4 < WKV_KR / 4; ++q4) {
+                    const float4 r4 = rr[q4], k4 = kk[q4], w4 = ww[q4];
+                    const float rv[4] = {r4.x, r4.y, r4.z, r4.w}, kv4[4] = {k4.x, k4.y, k4.z, k4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int ii = q4 * 4 + e;
+                        const float kv = kv4[e] * vj;
+                        part[e] = fmaf(rv[e], fmaf(ub[ii], kv, S[ii]), part[e]);
+                        S[ii] = fmaf(wv[e], S[ii], kv);
+                    }
                 }
+                float acc = (part[0] + part[1]) + (part[2] + part[3]);
                 for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, BN_WAVE);
                 if (p == 0 && owns) a.o[(size_t)(sr.row0 + c0 + tt) * (a.H * dv) + (size_t)head * dv + j] = acc;
             }
         }
+        __syncthreads();                                  // the chunk has been walked and the next one is staged
     }
 #pragma unroll
     for (int ii = 0; ii < WKV_KR; ++ii) {
-        const int i = p + P * ii;
+        const int i = p * WKV_KR + ii;
         if (owns && i < dk) S_g[(size_t)i * dv + j] = S[ii];
     }
     if (head == 0 && cb == 0) {                           // the step's last h of this sequence, for the next step's shift
@@ -167,21 +193,26 @@ __global__ void wkv_scan_kernel(WkvArgs a) {
     }
 }
 
-// The split of a head over threads and workgroups, as the launch below makes it (P, CB, TC, threads): the host side
-// asks for it to size nothing, only to say which head sizes are taken.
-static bool wkv_shape(int dk, int dv, int& P, int& CB, int& TC, int& threads) {
+// The split of a head over threads and workgroups (P, CB, TC, threads).  P follows from the head size alone (it fixes the
+// order of a column's sum); CB, the columns of a workgroup, is the largest that still gives the launch `want_wgs`
+// workgroups, down to one wave of threads, so that a prompt of one sequence spreads over the chip as a batch does.
+static bool wkv_shape(int dk, int dv, int groups, int& P, int& CB, int& TC, int& walkers, int& threads) {
     if (dk < 1 || dv < 1 || dk > WKV_MAX_DIM || dv > WKV_MAX_DIM) return false;
     P = 1;
     while (P * WKV_KR < dk) P <<= 1;                      // <= 16
-    CB = dv < 256 / P ? dv : 256 / P;
-    threads = ((CB * P + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
-    TC = P * WKV_KR <= 128 ? 16 : 8;
+    const int most = WKV_MAX_THREADS / P, least = BN_WAVE / P;          // columns of a full set of walkers, of one wave
+    CB = dv < most ? dv : most;
+    while (CB > least && (long long)groups * ((dv + CB - 1) / CB) < 256) CB = (CB + 1) / 2 < least ? least : (CB + 1) / 2;
+    walkers = ((CB * P + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
+    threads = walkers + (P >= 8 ? 128 : 64);              // and the staging waves
+    TC = 16;
+    while (TC > 1 && (size_t)2 * TC * (3 * P * WKV_KR + CB) * sizeof(float) > 48 * 1024) TC >>= 1;
     return true;
 }
 
 extern "C" int bn_wkv_supports(int dk, int dv) {
-    int P, CB, TC, th;
-    return wkv_shape(dk, dv, P, CB, TC, th) ? 1 : 0;
+    int P, CB, TC, wk, th;
+    return wkv_shape(dk, dv, 1, P, CB, TC, wk, th) ? 1 : 0;
 }
 
 extern "C" int bn_wkv_scan(int dtype, const void* r, int ldr, const void* k, int ldk, const void* v, int ldv, const void* d,
@@ -190,14 +221,14 @@ extern "C" int bn_wkv_scan(int dtype, const void* r, int ldr, const void* k, int
                            int H, int dk, int dv, int D, hipStream_t s) {
     WkvArgs a;
     int threads;
-    if (!wkv_shape(dk, dv, a.P, a.CB, a.TC, threads) || n_tiles <= 0 || H <= 0 || D <= 0) return BN_ERR_ARG;
+    if (n_tiles <= 0 || H <= 0 || D <= 0 || !wkv_shape(dk, dv, n_tiles * H, a.P, a.CB, a.TC, a.walkers, threads)) return BN_ERR_ARG;
     if (!r || !k || !v || !d || !w0 || !u || !o || !h || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
     if (state_stride < (long long)H * dk * dv + D) return BN_ERR_ARG;
     a.r = r; a.k = k; a.v = v; a.d = d; a.ldr = ldr; a.ldk = ldk; a.ldv = ldv; a.ldd = ldd;
     a.w0 = w0; a.u = u; a.o = o; a.h = h; a.state = state; a.state_stride = (size_t)state_stride;
     a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;
     a.H = H; a.dk = dk; a.dv = dv; a.D = D;
-    const size_t smem = (size_t)a.TC * (3 * a.P * WKV_KR + a.CB) * sizeof(float);
+    const size_t smem = (size_t)2 * a.TC * (3 * a.P * WKV_KR + a.CB) * sizeof(float);      // two staged chunks
     const dim3 grid(n_tiles, H, (dv + a.CB - 1) / a.CB);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(wkv_scan_kernel<float>, grid, dim3(threads), smem, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(wkv_scan_kernel<bf16>, grid, dim3(threads), smem, s, a);
@@ -238,32 +269,72 @@ extern "C" int bn_head_norm_gate(int dtype, void* y, const float* o, const void*
 
 // ---- min-GRU ------------------------------------------------------------------------------------------------------
 // zxg [T, ld]: the three projections side by side (update gate at 0, candidate at W, output gate at 2 W), without their
-// biases; a thread owns one channel of one sequence and walks its tokens.
+// biases.  A workgroup owns GRU_CH channels of one sequence.  Its tokens come in stages of GRU_TC: all threads load a
+// stage (the next one is asked for before the current one is walked), turn it into gate, candidate and silu(g) and
+// park those in shared memory; one thread a channel then walks the stage, S <- S + z (cand - S), and leaves S silu(g),
+// which all threads store.  The chain of a channel is the same operations in the same order whatever the step holds.
+#define GRU_CH 64
+#define GRU_TC 32
+#define GRU_THREADS 256
+#define GRU_PER_THREAD (GRU_CH * GRU_TC / GRU_THREADS)
+
 template <typename T>
-__global__ void mingru_scan_kernel(T* __restrict__ y, const T* __restrict__ zxg, int ld, const float* __restrict__ bz,
-                                   const float* __restrict__ bx, float* __restrict__ state, size_t state_stride,
-                                   const int* __restrict__ tiles, const int* __restrict__ seq_lens,
-                                   const int* __restrict__ slot_ids, int W) {
+__global__ __launch_bounds__(GRU_THREADS) void mingru_scan_kernel(T* __restrict__ y, const T* __restrict__ zxg, int ld,
+                                                                   const float* __restrict__ bz, const float* __restrict__ bx,
+                                                                   float* __restrict__ state, size_t state_stride,
+                                                                   const int* __restrict__ tiles, const int* __restrict__ seq_lens,
+                                                                   const int* __restrict__ slot_ids, int W) {
+    __shared__ float z_s[GRU_TC][GRU_CH], c_s[GRU_TC][GRU_CH], g_s[GRU_TC][GRU_CH];
     const SeqRange sr = seq_range(tiles, seq_lens, blockIdx.x);
     if (sr.n <= 0 || sr.pos0 < 0) return;
-    const int c = blockIdx.y * blockDim.x + threadIdx.x;
-    if (c >= W) return;
+    const int tid = threadIdx.x;
+    const int cc = tid % GRU_CH, t_first = tid / GRU_CH;            // this thread's channel and its first token of a stage
+    const int c = blockIdx.y * GRU_CH + cc;
+    const bool has = c < W;
     float* sp = state + (size_t)slot_ids[sr.seq] * state_stride + c;
-    float S = sr.pos0 > 0 ? *sp : 0.f;
-    const float biasz = bz ? bz[c] : 0.f, biasx = bx ? bx[c] : 0.f;
+    float S = (has && tid < GRU_CH && sr.pos0 > 0) ? *sp : 0.f;
+    const float biasz = (has && bz) ? bz[c] : 0.f, biasx = (has && bx) ? bx[c] : 0.f;
     const T* in = zxg + (size_t)sr.row0 * ld + c;
     T* out = y + (size_t)sr.row0 * W + c;
-#pragma unroll 4
-    for (int t = 0; t < sr.n; ++t) {
-        const float zp = to_f32(in[(size_t)t * ld]) + biasz;
-        const float cp = to_f32(in[(size_t)t * ld + W]) + biasx;
-        const float g = to_f32(in[(size_t)t * ld + 2 * W]);
-        const float z = 1.0f / (1.0f + expf(-zp));
-        const float cand = cp >= 0.f ? cp + 0.5f : 1.0f / (1.0f + expf(-cp));
-        S = fmaf(z, cand - S, S);                         // (1 - z) S + z cand
-        out[(size_t)t * W] = from_f32<T>(S * bn_unary_act(g, BN_UNARY_SILU));
+    float zr[GRU_PER_THREAD], cr[GRU_PER_THREAD], gr[GRU_PER_THREAD];
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < GRU_PER_THREAD; ++i) {
+            const int t = t0 + t_first + i * (GRU_THREADS / GRU_CH);
+            const bool in_range = has && t < sr.n;
+            zr[i] = in_range ? to_f32(in[(size_t)t * ld]) : 0.f;
+            cr[i] = in_range ? to_f32(in[(size_t)t * ld + W]) : 0.f;
+            gr[i] = in_range ? to_f32(in[(size_t)t * ld + 2 * W]) : 0.f;
+        }
+    };
+    fetch(0);
+    for (int t0 = 0; t0 < sr.n; t0 += GRU_TC) {
+#pragma unroll
+        for (int i = 0; i < GRU_PER_THREAD; ++i) {
+            const int tt = t_first + i * (GRU_THREADS / GRU_CH);
+            const float cp = cr[i] + biasx;
+            z_s[tt][cc] = 1.0f / (1.0f + expf(-(zr[i] + biasz)));
+            c_s[tt][cc] = cp >= 0.f ? cp + 0.5f : 1.0f / (1.0f + expf(-cp));
+            g_s[tt][cc] = bn_unary_act(gr[i], BN_UNARY_SILU);
+        }
+        __syncthreads();
+        if (t0 + GRU_TC < sr.n) fetch(t0 + GRU_TC);
+        const int nt = min(GRU_TC, sr.n - t0);
+        if (tid < GRU_CH) {
+            for (int tt = 0; tt < nt; ++tt) {
+                S = fmaf(z_s[tt][cc], c_s[tt][cc] - S, S);          // (1 - z) S + z cand
+                g_s[tt][cc] = S * g_s[tt][cc];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GRU_PER_THREAD; ++i) {
+            const int tt = t_first + i * (GRU_THREADS / GRU_CH);
+            if (has && tt < nt) out[(size_t)(t0 + tt) * W] = from_f32<T>(g_s[tt][cc]);
+        }
+        __syncthreads();
     }
-    *sp = S;
+    if (has && tid < GRU_CH) *sp = S;
 }
 
 extern "C" int bn_mingru_scan(int dtype, void* y, const void* zxg, int ld, const float* bz, const float* bx, float* state,
@@ -271,13 +342,12 @@ extern "C" int bn_mingru_scan(int dtype, void* y, const void* zxg, int ld, const
                               const int* slot_ids, int W, hipStream_t s) {
     if (n_tiles <= 0 || W <= 0 || ld < 3 * W || !y || !zxg || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
     if (state_stride < W) return BN_ERR_ARG;
-    const int threads = W >= 256 ? 256 : ((W + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
-    const dim3 grid(n_tiles, (W + threads - 1) / threads);
+    const dim3 grid(n_tiles, (W + GRU_CH - 1) / GRU_CH);
     if (dtype == BN_DT_F32)
-        hipLaunchKernelGGL(mingru_scan_kernel<float>, grid, dim3(threads), 0, s, (float*)y, (const float*)zxg, ld, bz, bx, state,
+        hipLaunchKernelGGL(mingru_scan_kernel<float>, grid, dim3(GRU_THREADS), 0, s, (float*)y, (const float*)zxg, ld, bz, bx, state,
                            (size_t)state_stride, tiles, seq_lens, slot_ids, W);
     else if (dtype == BN_DT_BF16)
-        hipLaunchKernelGGL(mingru_scan_kernel<bf16>, grid, dim3(threads), 0, s, (bf16*)y, (const bf16*)zxg, ld, bz, bx, state,
+        hipLaunchKernelGGL(mingru_scan_kernel<bf16>, grid, dim3(GRU_THREADS), 0, s, (bf16*)y, (const bf16*)zxg, ld, bz, bx, state,
                            (size_t)state_stride, tiles, seq_lens, slot_ids, W);
     else
         return BN_ERR_DTYPE;

@@ -15,6 +15,13 @@
 
 struct SeqRange { int seq, row0, n, pos0; };
 
+// A barrier of the workgroup that orders its shared memory only.  __syncthreads() also waits for everything that the wave
+// has asked from or sent to global memory; this one leaves loads and stores in flight (whoever needs a load's data waits
+// for it there), which is what lets a kernel ask for its next tokens before it walks the current ones.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ SeqRange seq_range(const int* tiles, const int* seq_lens, int idx) {
     SeqRange r;
     if (tiles) {
@@ -93,6 +100,39 @@ struct WkvArgs {
     int H, dk, dv, D, P, CB, TC, walkers;
 };
 
+// The sum over the P neighbouring lanes that share a column, every lane getting it: a butterfly whose steps of 1 and
+// 2 lanes are exchanges inside a group of four and whose steps of 4 and 8 lanes are mirrors of 8 and 16 lanes (after the
+// first two steps a group of four holds one value, so a mirror meets the same partner group as an exchange would).
+// Data-parallel moves inside a row of 16 lanes: no trip through shared memory.
+__device__ __forceinline__ float wkv_lane_sum(float v, int P) {
+    if (P >= 2) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));     // lanes 1 0 3 2
+    if (P >= 4) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));     // lanes 2 3 0 1
+    if (P >= 8) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));    // mirror of 8
+    if (P >= 16) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // mirror of 16
+    return v;
+}
+
+// One token of one column: o = sum_i r_i (S_i + u_i k_i v), then S_i <- w_i S_i + k_i v, over this thread's rows; the
+// sum in four partial sums and the lanes' butterfly.
+__device__ __forceinline__ float wkv_token(const float4 (&r4)[WKV_KR / 4], const float4 (&k4)[WKV_KR / 4],
+                                           const float4 (&w4)[WKV_KR / 4], float vj, const float (&ub)[WKV_KR],
+                                           float (&S)[WKV_KR], int P) {
+    float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q4 = 0; q4 < WKV_KR / 4; ++q4) {
+        const float rv[4] = {r4[q4].x, r4[q4].y, r4[q4].z, r4[q4].w}, kv4[4] = {k4[q4].x, k4[q4].y, k4[q4].z, k4[q4].w},
+                    wv[4] = {w4[q4].x, w4[q4].y, w4[q4].z, w4[q4].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ii = q4 * 4 + e;
+            const float kv = kv4[e] * vj;
+            part[e] = fmaf(rv[e], fmaf(ub[ii], kv, S[ii]), part[e]);
+            S[ii] = fmaf(wv[e], S[ii], kv);
+        }
+    }
+    return wkv_lane_sum((part[0] + part[1]) + (part[2] + part[3]), P);
+}
+
 template <typename T>
 __global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs a) {
     extern __shared__ __align__(16) float smem[];
@@ -126,26 +166,50 @@ __global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs
         float* w_s = k_s + TC * dkp;
         float* v_s = w_s + TC * dkp;
         const int nc = min(TC, sr.n - c0), lt = tid - n_walk, nl = nthreads - n_walk;
-        for (int idx = lt; idx < nc * dkp; idx += nl) {
-            const int tt = idx / dkp, i = idx - tt * dkp;
-            float rv = 0.f, kv = 0.f, wv = 0.f;
-            if (i < dk) {
+        // eight elements a turn, their loads asked for together (unconditional loads from clamped places: a load
+        // under a branch would make the compiler wait for each before the next)
+        const int total = nc * dkp;
+        for (int base = lt; base < total; base += 8 * nl) {
+            float rv[8], kv[8], dv4[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int idx = min(base + q * nl, total - 1);
+                const int tt = idx / dkp, i = min(idx - tt * dkp, dk - 1);
                 const size_t row = (size_t)(sr.row0 + c0 + tt), c = (size_t)head * dk + i;
-                rv = to_f32(reinterpret_cast<const T*>(a.r)[row * a.ldr + c]);
-                kv = to_f32(reinterpret_cast<const T*>(a.k)[row * a.ldk + c]);
-                wv = expf(-expf(to_f32(reinterpret_cast<const T*>(a.d)[row * a.ldd + c]) + a.w0[c]));
+                rv[q] = to_f32(reinterpret_cast<const T*>(a.r)[row * a.ldr + c]);
+                kv[q] = to_f32(reinterpret_cast<const T*>(a.k)[row * a.ldk + c]);
+                dv4[q] = to_f32(reinterpret_cast<const T*>(a.d)[row * a.ldd + c]) + a.w0[c];
             }
-            r_s[idx] = rv; k_s[idx] = kv; w_s[idx] = wv;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int idx = base + q * nl;
+                if (idx < total) {
+                    const bool in = idx % dkp < dk;
+                    r_s[idx] = in ? rv[q] : 0.f;
+                    k_s[idx] = in ? kv[q] : 0.f;
+                    w_s[idx] = in ? expf(-expf(dv4[q])) : 0.f;
+                }
+            }
         }
-        for (int idx = lt; idx < nc * CB; idx += nl) {
-            const int tt = idx / CB, col = cb * CB + (idx - tt * CB);
-            v_s[idx] = col < dv ? to_f32(reinterpret_cast<const T*>(a.v)[(size_t)(sr.row0 + c0 + tt) * a.ldv +
-                                                                          (size_t)head * dv + col]) : 0.f;
+        const int total_v = nc * CB;
+        for (int base = lt; base < total_v; base += 4 * nl) {
+            float vv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int idx = min(base + q * nl, total_v - 1);
+                const int tt = idx / CB, col = min(cb * CB + (idx - tt * CB), dv - 1);
+                vv[q] = to_f32(reinterpret_cast<const T*>(a.v)[(size_t)(sr.row0 + c0 + tt) * a.ldv + (size_t)head * dv + col]);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int idx = base + q * nl;
+                if (idx < total_v) v_s[idx] = cb * CB + idx % CB < dv ? vv[q] : 0.f;
+            }
         }
     };
 
     if (!walker) stage(0, 0);
-    __syncthreads();
+    lds_barrier();
     int b = 0;
     for (int c0 = 0; c0 < sr.n; c0 += TC, b ^= 1) {
         const int nc = min(TC, sr.n - c0);
@@ -156,30 +220,35 @@ __global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs
             const float* k_s = r_s + TC * dkp;
             const float* w_s = k_s + TC * dkp;
             const float* v_s = w_s + TC * dkp;
-            for (int tt = 0; tt < nc; ++tt) {
-                const float vj = v_s[tt * CB + jl];
-                const float4* rr = reinterpret_cast<const float4*>(r_s + tt * dkp + p * WKV_KR);
-                const float4* kk = reinterpret_cast<const float4*>(k_s + tt * dkp + p * WKV_KR);
-                const float4* ww = reinterpret_cast<const float4*>(w_s + tt * dkp + p * WKV_KR);
-                float part[4] = {0.f, 0.f, 0.f, 0.f};
+            // two tokens a turn: both tokens' rows are asked for before the first is used, so the second's way from
+            // shared memory is covered by the first's arithmetic
+            for (int tt = 0; tt < nc; tt += 2) {
+                const bool two = tt + 1 < nc;
+                const int t1 = two ? tt + 1 : tt;
+                float4 ra[WKV_KR / 4], ka[WKV_KR / 4], wa[WKV_KR / 4], rb[WKV_KR / 4], kb[WKV_KR / 4], wb[WKV_KR / 4];
 #pragma unroll
                 for (int q4 = 0; q4 < WKV_KR / 4; ++q4) {
-                    const float4 r4 = rr[q4], k4 = kk[q4], w4 = ww[q4];
-                    const float rv[4] = {r4.x, r4.y, r4.z, r4.w}, kv4[4] = {k4.x, k4.y, k4.z, k4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int ii = q4 * 4 + e;
-                        const float kv = kv4[e] * vj;
-                        part[e] = fmaf(rv[e], fmaf(ub[ii], kv, S[ii]), part[e]);
-                        S[ii] = fmaf(wv[e], S[ii], kv);
-                    }
+                    ra[q4] = reinterpret_cast<const float4*>(r_s + tt * dkp + p * WKV_KR)[q4];
+                    ka[q4] = reinterpret_cast<const float4*>(k_s + tt * dkp + p * WKV_KR)[q4];
+                    wa[q4] = reinterpret_cast<const float4*>(w_s + tt * dkp + p * WKV_KR)[q4];
                 }
-                float acc = (part[0] + part[1]) + (part[2] + part[3]);
-                for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, BN_WAVE);
-                if (p == 0 && owns) a.o[(size_t)(sr.row0 + c0 + tt) * (a.H * dv) + (size_t)head * dv + j] = acc;
+                const float va = v_s[tt * CB + jl];
+#pragma unroll
+                for (int q4 = 0; q4 < WKV_KR / 4; ++q4) {
+                    rb[q4] = reinterpret_cast<const float4*>(r_s + t1 * dkp + p * WKV_KR)[q4];
+                    kb[q4] = reinterpret_cast<const float4*>(k_s + t1 * dkp + p * WKV_KR)[q4];
+                    wb[q4] = reinterpret_cast<const float4*>(w_s + t1 * dkp + p * WKV_KR)[q4];
+                }
+                const float vb = v_s[t1 * CB + jl];
+                const float acc_a = wkv_token(ra, ka, wa, va, ub, S, P);
+                if (p == 0 && owns) a.o[(size_t)(sr.row0 + c0 + tt) * (a.H * dv) + (size_t)head * dv + j] = acc_a;
+                if (two) {
+                    const float acc_b = wkv_token(rb, kb, wb, vb, ub, S, P);
+                    if (p == 0 && owns) a.o[(size_t)(sr.row0 + c0 + t1) * (a.H * dv) + (size_t)head * dv + j] = acc_b;
+                }
             }
         }
-        __syncthreads();                                  // the chunk has been walked and the next one is staged
+        lds_barrier();                                    // the chunk has been walked and the next one is staged
     }
 #pragma unroll
     for (int ii = 0; ii < WKV_KR; ++ii) {
@@ -204,9 +273,9 @@ static bool wkv_shape(int dk, int dv, int groups, int& P, int& CB, int& TC, int&
     CB = dv < most ? dv : most;
     while (CB > least && (long long)groups * ((dv + CB - 1) / CB) < 256) CB = (CB + 1) / 2 < least ? least : (CB + 1) / 2;
     walkers = ((CB * P + BN_WAVE - 1) / BN_WAVE) * BN_WAVE;
-    threads = walkers + (P >= 8 ? 128 : 64);              // and the staging waves
-    TC = 16;
-    while (TC > 1 && (size_t)2 * TC * (3 * P * WKV_KR + CB) * sizeof(float) > 48 * 1024) TC >>= 1;
+    threads = walkers + 128;                              // and the staging waves
+    TC = 32;                                              // the longest chunk whose two buffers fit beside each other
+    while (TC > 4 && (size_t)2 * TC * (3 * P * WKV_KR + CB) * sizeof(float) > 60 * 1024) TC >>= 1;
     return true;
 }
 
@@ -274,7 +343,7 @@ extern "C" int bn_head_norm_gate(int dtype, void* y, const float* o, const void*
 // park those in shared memory; one thread a channel then walks the stage, S <- S + z (cand - S), and leaves S silu(g),
 // which all threads store.  The chain of a channel is the same operations in the same order whatever the step holds.
 #define GRU_CH 64
-#define GRU_TC 32
+#define GRU_TC 64
 #define GRU_THREADS 256
 #define GRU_PER_THREAD (GRU_CH * GRU_TC / GRU_THREADS)
 
@@ -294,17 +363,18 @@ __global__ __launch_bounds__(GRU_THREADS) void mingru_scan_kernel(T* __restrict_
     float* sp = state + (size_t)slot_ids[sr.seq] * state_stride + c;
     float S = (has && tid < GRU_CH && sr.pos0 > 0) ? *sp : 0.f;
     const float biasz = (has && bz) ? bz[c] : 0.f, biasx = (has && bx) ? bx[c] : 0.f;
-    const T* in = zxg + (size_t)sr.row0 * ld + c;
+    const T* in = zxg + (size_t)sr.row0 * ld + (has ? c : 0);
     T* out = y + (size_t)sr.row0 * W + c;
     float zr[GRU_PER_THREAD], cr[GRU_PER_THREAD], gr[GRU_PER_THREAD];
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < GRU_PER_THREAD; ++i) {
-            const int t = t0 + t_first + i * (GRU_THREADS / GRU_CH);
-            const bool in_range = has && t < sr.n;
-            zr[i] = in_range ? to_f32(in[(size_t)t * ld]) : 0.f;
-            cr[i] = in_range ? to_f32(in[(size_t)t * ld + W]) : 0.f;
-            gr[i] = in_range ? to_f32(in[(size_t)t * ld + 2 * W]) : 0.f;
+            // unconditional loads from clamped places (a load under a branch is waited for where it stands); what a
+            // thread without a channel or a token loads is never stored
+            const int t = min(t0 + t_first + i * (GRU_THREADS / GRU_CH), sr.n - 1);
+            zr[i] = to_f32(in[(size_t)t * ld]);
+            cr[i] = to_f32(in[(size_t)t * ld + W]);
+            gr[i] = to_f32(in[(size_t)t * ld + 2 * W]);
         }
     };
     fetch(0);
@@ -317,22 +387,30 @@ __global__ __launch_bounds__(GRU_THREADS) void mingru_scan_kernel(T* __restrict_
             c_s[tt][cc] = cp >= 0.f ? cp + 0.5f : 1.0f / (1.0f + expf(-cp));
             g_s[tt][cc] = bn_unary_act(gr[i], BN_UNARY_SILU);
         }
-        __syncthreads();
+        lds_barrier();
         if (t0 + GRU_TC < sr.n) fetch(t0 + GRU_TC);
         const int nt = min(GRU_TC, sr.n - t0);
         if (tid < GRU_CH) {
-            for (int tt = 0; tt < nt; ++tt) {
-                S = fmaf(z_s[tt][cc], c_s[tt][cc] - S, S);          // (1 - z) S + z cand
-                g_s[tt][cc] = S * g_s[tt][cc];
+            for (int tt = 0; tt < nt; tt += 8) {                    // eight tokens' values at once, then their chain
+                float z8[8], c8[8], g8[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { z8[i] = z_s[tt + i][cc]; c8[i] = c_s[tt + i][cc]; g8[i] = g_s[tt + i][cc]; }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (tt + i < nt) {
+                        S = fmaf(z8[i], c8[i] - S, S);              // (1 - z) S + z cand
+                        g_s[tt + i][cc] = S * g8[i];
+                    }
+                }
             }
         }
-        __syncthreads();
+        lds_barrier();
 #pragma unroll
         for (int i = 0; i < GRU_PER_THREAD; ++i) {
             const int tt = t_first + i * (GRU_THREADS / GRU_CH);
             if (has && tt < nt) out[(size_t)(t0 + tt) * W] = from_f32<T>(g_s[tt][cc]);
         }
-        __syncthreads();
+        lds_barrier();
     }
     if (has && tid < GRU_CH) *sp = S;
 }

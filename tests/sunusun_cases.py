@@ -26,6 +26,11 @@ CONFIGS = {
         _wkv(3, 20, 5, ff=50),
         _par(4, 2, 16, 24, 0.31, 0.2, 3, 40, ff=72, weights_of=0),
         _wkv(3, 20, 5, ff=50, weights_of=2)]),
+    # recurrent layers alone (no keys or values anywhere: a cache without pages) and parallel layers alone
+    "R": dict(architecture="Sunusun", vocab=50, width=40, norm=dict(eps=1e-5), logit_scale=0.7, layers=[
+        _wkv(2, 16, 3, ff=48), _wkv(5, 8, 2), _wkv(2, 16, 3, ff=48, weights_of=0)]),
+    "S": dict(architecture="Sunusun", vocab=70, width=24, norm=dict(eps=1e-5), logit_scale=1.5, layers=[
+        _par(8, 1, 4, 2, 0.6, -0.2, 9, 8, ff=30), _par(2, 2, 32, 32, 0.2, 0.4, 100, 64)]),
     "Q": dict(architecture="Sunusun", vocab=131, width=48, norm=dict(eps=1e-6), logit_scale=1.0, layers=[
         _wkv(1, 32, 4, ff=64, weights_of=2),
         _par(3, 3, 8, 6, 0.9, 0.5, 1, 33),

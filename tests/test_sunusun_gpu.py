@@ -428,6 +428,35 @@ def test_unequal_batches_and_slots_used_again(folders, name, dtype, graphs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_prompt_steps_replayed_from_graphs(folders, name, dtype):
+    """Prompt steps of one size run eagerly the first time, are recorded the second time and replayed afterwards, with
+    other sequences in other slots each time: every one of them against the plain implementation, and the state that a
+    recorded step left is what the tokens decoded behind it go on from."""
+    import bitnet_c_amd as bn
+    folder = folders(name, dtype)
+    eng = engine(folder, dtype)
+    vocab = CONFIGS[name]["vocab"]
+    keep = eng.new_sequence()                      # a live neighbour, so that later sequences get other slots
+    eng.step([bn.StepEntry(keep, tokens_of(vocab, 1, 9), [])])
+    for i in range(5):
+        reqs = [tokens_of(vocab, 300 + 10 * i + k, n) for k, n in enumerate((70 + i, 20 - i))]
+        slots = [eng.new_sequence() for _ in reqs]
+        out = eng.step([bn.StepEntry(s, r[:-3], [0, len(r) - 4]) for s, r in zip(slots, reqs)])
+        tail = [eng.step([bn.StepEntry(s, [r[t]], [0]) for s, r in zip(slots, reqs)]) for t in (-3, -2, -1)]
+        for k, r in enumerate(reqs):
+            want = plain(folder, r)
+            close(out[2 * k:2 * k + 2], want[[0, len(r) - 4]], dtype)
+            close(torch.cat([t[k:k + 1] for t in tail]), want[-3:], dtype)
+        if i % 2:
+            eng.release(slots[0])
+        else:
+            eng.release(slots[1])
+    assert not eng.prompt_graphs or eng.graphs_built >= 2          # a prompt step and the decode steps were recorded
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_a_step_that_mixes_single_tokens_and_portions(folders, dtype):
     import bitnet_c_amd as bn
     folder = folders("P", dtype)

@@ -43,14 +43,20 @@ __global__ void token_shift_kernel(T* __restrict__ out, const T* __restrict__ h,
                                    const int* __restrict__ seq_index, const int* __restrict__ slot_ids, int T_rows, int D,
                                    int n_mix) {
     const int t = blockIdx.x;
-    const int pos = positions[t];
+    const int pos = positions[t], seq = seq_index[t];
+    const int before = t > 0 ? t - 1 : 0;
+    const int pos_b = positions[before], seq_b = seq_index[before], slot = slot_ids[seq];     // all asked for together
     const T* cur = h + (size_t)t * D;
-    const bool inside = t > 0 && pos > 0 && seq_index[t - 1] == seq_index[t] && positions[t - 1] == pos - 1;
-    const T* prev_row = inside ? h + (size_t)(t - 1) * D : nullptr;
-    const float* prev_state = (!inside && pos > 0) ? state + (size_t)slot_ids[seq_index[t]] * state_stride : nullptr;
+    const bool inside = t > 0 && pos > 0 && seq_b == seq && pos_b == pos - 1;
+    // both candidates for the previous row are loaded, from places that exist, and one is chosen: a load under a
+    // branch would be waited for where it stands, element after element
+    const T* prev_row = h + (size_t)(inside ? t - 1 : t) * D;
+    const float* prev_state = state + (size_t)slot * state_stride;
+#pragma unroll 4
     for (int e = threadIdx.x; e < D; e += blockDim.x) {
         const float c = to_f32(cur[e]);
-        const float p = prev_row ? to_f32(prev_row[e]) : (prev_state ? prev_state[e] : 0.f);
+        const float pr = to_f32(prev_row[e]), ps = prev_state[e];
+        const float p = inside ? pr : (pos > 0 ? ps : 0.f);
         const float d = p - c;
         for (int s = 0; s < n_mix; ++s)
             out[((size_t)s * T_rows + t) * D + e] = from_f32<T>(pos >= 0 ? fmaf(d, mu[(size_t)s * D + e], c) : 0.f);
@@ -94,7 +100,7 @@ struct WkvArgs {
     const float* u;           // [H * dk] the bonus of the current token
     float* o;                 // [T, H * dv] float32
     const void* h;            // [T, D]: the mixer's input, whose last row of every sequence becomes the state's copy
-    float* state;             // [slots, state_stride]: S as [H][dk][dv], then D values of the last h
+    float* state;             // [slots, state_stride]: S per head in the walkers' order (wkv_state_at), then D values of the last h
     size_t state_stride;
     const int* tiles; const int* seq_lens; const int* slot_ids;
     int H, dk, dv, D, P, CB, TC, walkers;
@@ -149,14 +155,15 @@ __global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs
     const bool owns = walker && jl < CB && j < dv;
     const int buf_floats = TC * (3 * dkp + CB);           // one staged chunk: r, k, w as [TC][dkp], then v as [TC][CB]
 
-    float* S_g = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * dk * dv;
+    // A head's state lies in the order in which the walkers hold it: element (row p WKV_KR + ii, column j) at
+    // (ii dv + j) P + p, so that the lanes of a wave, p fastest and then the columns, read and write runs of memory.
+    float* S_g = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * dkp * dv;
     float S[WKV_KR], ub[WKV_KR];
 #pragma unroll
     for (int ii = 0; ii < WKV_KR; ++ii) {
         const int i = p * WKV_KR + ii;
-        const bool in = owns && i < dk;
-        S[ii] = (in && sr.pos0 > 0) ? S_g[(size_t)i * dv + j] : 0.f;
-        ub[ii] = in ? a.u[(size_t)head * dk + i] : 0.f;
+        S[ii] = (owns && sr.pos0 > 0) ? S_g[((size_t)ii * dv + j) * P + p] : 0.f;        // rows beyond dk hold zeros
+        ub[ii] = (owns && i < dk) ? a.u[(size_t)head * dk + i] : 0.f;
     }
 
     // the staging threads' work: chunk c0 into buffer b
@@ -251,12 +258,10 @@ __global__ __launch_bounds__(WKV_MAX_THREADS + 128) void wkv_scan_kernel(WkvArgs
         lds_barrier();                                    // the chunk has been walked and the next one is staged
     }
 #pragma unroll
-    for (int ii = 0; ii < WKV_KR; ++ii) {
-        const int i = p * WKV_KR + ii;
-        if (owns && i < dk) S_g[(size_t)i * dv + j] = S[ii];
-    }
+    for (int ii = 0; ii < WKV_KR; ++ii)
+        if (owns) S_g[((size_t)ii * dv + j) * P + p] = S[ii];
     if (head == 0 && cb == 0) {                           // the step's last h of this sequence, for the next step's shift
-        float* hp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)a.H * dk * dv;
+        float* hp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)a.H * dkp * dv;
         const T* last = reinterpret_cast<const T*>(a.h) + (size_t)(sr.row0 + sr.n - 1) * a.D;
         for (int e = tid; e < a.D; e += nthreads) hp[e] = to_f32(last[e]);
     }
@@ -284,6 +289,12 @@ extern "C" int bn_wkv_supports(int dk, int dv) {
     return wkv_shape(dk, dv, 1, P, CB, TC, wk, th) ? 1 : 0;
 }
 
+// float32 values of one head's state: dk rounded up to the rows that the walkers hold (a power of two times WKV_KR), times dv
+extern "C" int bn_wkv_state_floats(int dk, int dv) {
+    int P, CB, TC, wk, th;
+    return wkv_shape(dk, dv, 1, P, CB, TC, wk, th) ? P * WKV_KR * dv : 0;
+}
+
 extern "C" int bn_wkv_scan(int dtype, const void* r, int ldr, const void* k, int ldk, const void* v, int ldv, const void* d,
                            int ldd, const float* w0, const float* u, float* o, const void* h, float* state,
                            long long state_stride, const int* tiles, int n_tiles, const int* seq_lens, const int* slot_ids,
@@ -292,7 +303,7 @@ extern "C" int bn_wkv_scan(int dtype, const void* r, int ldr, const void* k, int
     int threads;
     if (n_tiles <= 0 || H <= 0 || D <= 0 || !wkv_shape(dk, dv, n_tiles * H, a.P, a.CB, a.TC, a.walkers, threads)) return BN_ERR_ARG;
     if (!r || !k || !v || !d || !w0 || !u || !o || !h || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
-    if (state_stride < (long long)H * dk * dv + D) return BN_ERR_ARG;
+    if (state_stride < (long long)H * a.P * WKV_KR * dv + D) return BN_ERR_ARG;
     a.r = r; a.k = k; a.v = v; a.d = d; a.ldr = ldr; a.ldk = ldk; a.ldv = ldv; a.ldd = ldd;
     a.w0 = w0; a.u = u; a.o = o; a.h = h; a.state = state; a.state_stride = (size_t)state_stride;
     a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;

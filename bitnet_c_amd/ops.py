@@ -58,6 +58,7 @@ _SIGNATURES = {
         "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
                            c_int, c_int, c_void_p],
         "bn_wkv_supports": [c_int, c_int],
+        "bn_wkv_state_floats": [c_int, c_int],
         "bn_wkv_scan": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                         c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                         c_int, c_void_p],
@@ -1473,11 +1474,26 @@ def wkv_supported(dk: int, dv: int) -> bool:
     return 1 <= dk <= WKV_MAX_DIM and 1 <= dv <= WKV_MAX_DIM
 
 
+WKV_ROWS_PER_THREAD = _build.header_constant("WKV_KR", "state_mixers.hip")
+
+
+def wkv_state_floats(H: int, dk: int, dv: int) -> int:
+    """float32 values of the matrix states of H heads as wkv_scan keeps them: the dk rows of a head are rounded up to a
+    power of two times the rows a thread holds (the kernel spreads a column's rows over that many neighbouring lanes and
+    stores the state in the lanes' order, which no one else reads)."""
+    if not wkv_supported(dk, dv):
+        raise KernelError(f"wkv: head sizes up to {WKV_MAX_DIM}, got {dk} x {dv}")
+    p = 1
+    while p * WKV_ROWS_PER_THREAD < dk:
+        p *= 2
+    return H * p * WKV_ROWS_PER_THREAD * dv
+
+
 def wkv_scan(r, k, v, d, w0, u, h, state, slot_ids, H: int, dk: int, dv: int, *, tiles=None, seq_lens=None) -> torch.Tensor:
     """The wkv recurrence over every sequence of a step; float32 [T, H dv].  r, k, d: [T, H dk] (rows contiguous, any row
     stride), v: [T, H dv], in the activations' type; w0, u: float32 [H dk] (the decay's offset, the current token's
-    bonus); h [T, D]: the mixer's input.  state [slots, >= H dk dv + D] float32: S per head as [dk, dv], then the last
-    h, both updated in place.  Per head, in float32:
+    bonus); h [T, D]: the mixer's input.  state [slots, >= wkv_state_floats(H, dk, dv) + D] float32: the heads' matrices
+    in the kernel's own order, then the last h, both updated in place.  Per head, in float32:
         w_t = exp(-exp(d_t + w0));  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T."""
     require_gpu()
     _dev(h, "h", dims=2)
@@ -1494,7 +1510,7 @@ def wkv_scan(r, k, v, d, w0, u, h, state, slot_ids, H: int, dk: int, dv: int, *,
             raise KernelError(f"wkv_scan: {nm} must hold {H * dk} float32 values")
     if not h.is_contiguous():
         raise KernelError("wkv_scan: h must be contiguous")
-    stride = _state_rows(state, H * dk * dv + D, "wkv_scan")
+    stride = _state_rows(state, wkv_state_floats(H, dk, dv) + D, "wkv_scan")
     _dev(slot_ids, "slot_ids", torch.int32, 1)
     tl, n_tiles, sl = _seq_args(tiles, seq_lens, "wkv_scan")
     o = torch.empty((T, H * dv), dtype=torch.float32, device=h.device)

@@ -51,6 +51,10 @@ class WKV(Part):
     def inner(self):
         return self.H * self.hs
 
+    @property
+    def state_floats(self):
+        return ops.wkv_state_floats(self.H, self.hs, self.hs)
+
     def tensors(self):
         D, A = self.hidden, self.inner
         t = {f"mu_{s}": ParamSpec((D,), "normal") for s in self.MIXES}
@@ -72,13 +76,13 @@ class WKV(Part):
         return [self.r, self.k, self.v, self.g, self.o]
 
     def cache_need(self) -> CacheNeed:
-        # per head a [head_dim, head_dim] matrix, then the last input row
-        return CacheNeed(state=StateNeed((self.inner * self.hs + self.hidden,), torch.float32, device_addressed=True))
+        # per head a [head_dim, head_dim] matrix (in the kernel's own order and rounding of its rows), then the last input row
+        return CacheNeed(state=StateNeed((self.state_floats + self.hidden,), torch.float32, device_addressed=True))
 
     def forward(self, h, ctx, kv):
         H, hs = self.H, self.hs
         state = kv.state
-        mixes = ops.token_shift(h, self.mu, state[:, self.inner * hs:], ctx.positions, ctx.seq_index, ctx.slot_ids)
+        mixes = ops.token_shift(h, self.mu, state[:, self.state_floats:], ctx.positions, ctx.seq_index, ctx.slot_ids)
         r, k, v, g = self.r(mixes[0]), self.k(mixes[1]), self.v(mixes[2]), self.g(mixes[3])
         low = self.w1(mixes[4])
         ops.unary_act(low, "tanh", out=low)

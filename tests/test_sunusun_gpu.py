@@ -124,7 +124,8 @@ def test_wkv_pieces_alone(dtype, H, d):
     dd = [(-1.0 + torch.randn(n, A, generator=g)).to(dtype) for n in lens]
     gate = [torch.randn(n, A, generator=g).to(dtype) for n in lens]
     w0, u, nw = 0.3 * torch.randn(A, generator=g), 0.5 * torch.randn(A, generator=g), 1 + 0.1 * torch.randn(A, generator=g)
-    state = torch.zeros(4, A * d + D, dtype=torch.float32, device=dev)
+    n_state = ops.wkv_state_floats(H, d, d)          # the heads' matrices, rows rounded up as the kernel holds them
+    state = torch.zeros(4, n_state + D, dtype=torch.float32, device=dev)
     state[3] = 7.0
     slots = torch.tensor([2, 0], dtype=torch.int32, device=dev)
 
@@ -134,7 +135,7 @@ def test_wkv_pieces_alone(dtype, H, d):
         pos, seq, tiles = _seq_tensors(lengths, starts, dev)
         cat = lambda xs: torch.cat([x[p] for x, p in zip(xs, parts)]).to(dev).contiguous()
         h = cat(hs)
-        mixes = ops.token_shift(h, mu.to(dev), state[:, A * d:], pos, seq, slots)
+        mixes = ops.token_shift(h, mu.to(dev), state[:, n_state:], pos, seq, slots)
         o = ops.wkv_scan(cat(r), cat(k), cat(v), cat(dd), w0.to(dev), u.to(dev), h, state, slots, H, d, d, tiles=tiles)
         y = ops.head_norm_gate(o, cat(gate), nw.to(dev), H, d, eps)
         return mixes, o, y
@@ -157,7 +158,7 @@ def test_wkv_pieces_alone(dtype, H, d):
         assert rel_err(got_o, want_o.reshape(n, A)) < 2e-5            # float32 whatever the activations' type
         close(got_y, want_y, dtype)
     assert bool((state[3] == 7.0).all()) and bool((state[1] == 0).all())
-    assert torch.equal(state[0, A * d:].cpu(), hs[1][-1].float())      # the last input row, for the next step's shift
+    assert torch.equal(state[0, n_state:].cpu(), hs[1][-1].float())      # the last input row, for the next step's shift
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

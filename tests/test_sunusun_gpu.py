@@ -543,3 +543,49 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
             assert float(logits[i].max() - logits[i, tok]) <= 4e-2 * rms
     llm.engine.cache.check()
     assert llm.engine.cache.live_slots() == []
+
+
+def test_command_line_and_trace_replay(folders, tmp_path):
+    """The command line generates from a Sunusun folder (also one that it writes itself from a configuration file, with
+    random weights), and the trace replay program steps one through portions and single tokens."""
+    import subprocess
+    import sys
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = folders("P", torch.float32)
+    cfg, W = ps.read_config(folder), ps.read_weights(folder)
+    prompt = [3, 1, 4, 1, 5, 9, 2, 6]
+    want = ps.generate(cfg, W, prompt, 6)
+    base = [sys.executable, os.path.join(root, "bin", "bitnet"), folder, "--prompt-token-ids", ",".join(map(str, prompt)),
+            "-n", "6", "--repeat-penalty", "1.0", "--fp32", "--token-ids", "--quiet"]
+    for extra in ([], ["--no-prefill"]):
+        p = subprocess.run(base + extra, capture_output=True, text=True, timeout=300)
+        assert p.returncode == 0, p.stderr[-1500:]
+        ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+        assert [int(x) for x in ids.split(",")] == want, extra
+    conf = tmp_path / "conf.json"
+    conf.write_text(json.dumps(CONFIGS["R"]))
+    made = str(tmp_path / "made")
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "bitnet"), made, "--random", str(conf), "--seed", "4",
+                        "--prompt-token-ids", "1,2,3", "-n", "4", "--fp32", "--token-ids", "--quiet", "--repeat-penalty", "1.0"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    ids = [l for l in p.stderr.splitlines() if l and l[0].isdigit()][0]
+    assert [int(x) for x in ids.split(",")] == ps.generate(ps.read_config(made), ps.read_weights(made), [1, 2, 3], 4)
+    # trace replay: two requests, the first in two portions, then both token by token; logits at the wanted places
+    a, b = tokens_of(97, 1, 40), tokens_of(97, 2, 7)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[30:38], "want": [7]}, {"id": "b", "tokens": b[:5], "want": [4]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[38:39], "want": [0]}, {"id": "b", "tokens": b[5:6], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[39:], "want": [0]}, {"id": "b", "tokens": b[6:], "want": [0]}], "end": ["a", "b"]}]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-1500:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    la, lb = ps.forward(cfg, W, a), ps.forward(cfg, W, b)
+    want_rows = {0: la[[0, 29]], 1: torch.stack([la[37], lb[4]]), 2: la[38:39], 3: torch.stack([la[39], lb[6]])}
+    for i, w in want_rows.items():
+        got = torch.from_numpy(np.fromfile(str(out / f"{i}.f32"), dtype="<f4").reshape(-1, 97))
+        close(got, w, torch.float32)

@@ -31,6 +31,11 @@ CONFIGS = {
         _wkv(2, 16, 3, ff=48), _wkv(5, 8, 2), _wkv(2, 16, 3, ff=48, weights_of=0)]),
     "S": dict(architecture="Sunusun", vocab=70, width=24, norm=dict(eps=1e-5), logit_scale=1.5, layers=[
         _par(8, 1, 4, 2, 0.6, -0.2, 9, 8, ff=30), _par(2, 2, 32, 32, 0.2, 0.4, 100, 64)]),
+    # the head sizes of real models (64 for the recurrence, 64 and 128 for attention: sizes at which other kernels of the
+    # library would claim bf16 pages of another order), a parallel layer first, a feed-forward narrower than the width
+    "T": dict(architecture="Sunusun", vocab=211, width=128, norm=dict(eps=1e-6), logit_scale=0.25, layers=[
+        _par(4, 2, 64, 64, 0.125, 0.3, 16, 96, ff=64), _wkv(2, 64, 16, ff=192), _par(2, 1, 128, 32, 0.09, 0.2, 50, 128),
+        _wkv(2, 64, 16, ff=192, weights_of=1)]),
     "Q": dict(architecture="Sunusun", vocab=131, width=48, norm=dict(eps=1e-6), logit_scale=1.0, layers=[
         _wkv(1, 32, 4, ff=64, weights_of=2),
         _par(3, 3, 8, 6, 0.9, 0.5, 1, 33),

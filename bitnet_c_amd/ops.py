@@ -1107,7 +1107,10 @@ def pair_tiles(rows: list) -> list:
 DECODE_TARGET_WGS = int(os.environ.get("BITNET_DECODE_WGS", "256"))
 
 
-def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
+VECTOR_DECODE_TARGET_WGS = int(os.environ.get("BITNET_VECTOR_DECODE_WGS", "1024"))     # see decode_splits
+
+
+def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None, target_wgs: int = 0):
     """(n_splits, chunk): how the keys of a decode step are cut so that the launch fills the
     chip.  A function of the batch's shape and of max_len alone.  A float32 cache is cut in runs of F32_FOLD_KEYS
     positions whatever the batch: both forms of the float32 kernel sum a query's keys run by run and fold the runs in
@@ -1120,7 +1123,10 @@ def decode_splits(n_seqs: int, H: int, Hkv: int, max_len: int, dtype=None):
     pages = max(1, (max_len + PAGE - 1) // PAGE)
     # about DECODE_TARGET_WGS workgroups, but no split shorter than SPLIT_MIN_PAGES pages: below that the merging costs
     # more than the parallelism gains (measured at batch 1, 8 and 64 of the 8B shape)
-    want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (DECODE_TARGET_WGS + wgs - 1) // wgs))
+    # target_wgs: another aim than DECODE_TARGET_WGS (the vector kernel's workgroups are small, several fit on a CU and
+    # hide each other's waits: VECTOR_DECODE_TARGET_WGS)
+    target = target_wgs or DECODE_TARGET_WGS
+    want = max(1, min(pages // SPLIT_MIN_PAGES, 64, (target + wgs - 1) // wgs))
     chunk = ((pages + want - 1) // want) * PAGE
     n_splits = (pages * PAGE + chunk - 1) // chunk
     return n_splits, chunk

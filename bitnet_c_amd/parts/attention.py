@@ -137,7 +137,8 @@ class Attention(Part):
         out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
         bias = (self.dist_a, self.dist_b) if self.distance_bias else None
         if ctx.is_decode:
-            n_splits, chunk = (1, 0) if self.window else ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype)
+            n_splits, chunk = (1, 0) if self.window else ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype,
+                                                                           target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=False, blocked=False,

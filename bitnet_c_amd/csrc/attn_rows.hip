@@ -255,9 +255,18 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             if (a.v_transposed) {
                 const T* vt = reinterpret_cast<const T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * vd * BN_PAGE +
                               (j0 % BN_PAGE);
-                for (int idx = tid; idx < KT * vd; idx += ATT_THREADS) {
-                    const int d = idx / KT, j = idx - d * KT;
-                    v_s[j * vstride + d] = (j0 + j < hi) ? vt[(size_t)d * BN_PAGE + j] : from_f32<T>(0.f);
+                // 16 bytes of one value column (8 or 4 consecutive positions) a load; neighbouring threads take
+                // neighbouring columns, so that their stores into the staged rows meet no bank twice
+                constexpr int EPV = 16 / (int)sizeof(T);
+                struct Group { T e[EPV]; };
+                for (int idx = tid; idx < (KT / EPV) * vd; idx += ATT_THREADS) {
+                    const int jc = idx / vd, d = idx - jc * vd;
+                    const Group w = __builtin_bit_cast(Group, *reinterpret_cast<const uint4*>(vt + (size_t)d * BN_PAGE + jc * EPV));
+#pragma unroll
+                    for (int q = 0; q < EPV; ++q) {
+                        const int j = jc * EPV + q;
+                        v_s[j * vstride + d] = (j0 + j < hi) ? w.e[q] : from_f32<T>(0.f);
+                    }
                 }
             }
         }

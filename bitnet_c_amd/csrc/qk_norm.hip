@@ -7,7 +7,8 @@
 //   k_g <- k_g / sqrt(mean(k_g^2) + eps) * wk          -> page of position p
 //   v_g                                                 -> page of position p
 //
-// Pages hold a row per position ("rows" layout): keys [page, kv head, BN_PAGE, hs], values [page, kv head, BN_PAGE, vd].
+// Pages hold a row per position for the keys, [page, kv head, BN_PAGE, hs]; the values lie the same way ("rows" layout,
+// [page, kv head, BN_PAGE, vd]) or transposed ([page, kv head, vd, BN_PAGE]), as the caller says.
 #include "common.h"
 #include <math.h>
 
@@ -21,6 +22,7 @@ struct QkNormArgs {
     const float* wq;          // [hs] or null: no norm
     const float* wk;
     int ld, bt_stride, H, Hkv, hs, vd;
+    int v_transposed;         // the values' pages are [page, kv head, vd, BN_PAGE]
     float eps, temp_coef;
     int temp_every;           // <= 0: no temperature
 };
@@ -62,15 +64,20 @@ __global__ __launch_bounds__(BN_WAVE) void qk_norm_store_kernel(QkNormArgs a) {
         const int kvh = head - a.H - a.Hkv;
         const T* v = row + (size_t)(a.H + a.Hkv) * a.hs + (size_t)kvh * a.vd;
         const int page = a.block_table[(size_t)a.seq_index[t] * a.bt_stride + pos / BN_PAGE];
-        T* dst = reinterpret_cast<T*>(a.v_pages) + (((size_t)page * a.Hkv + kvh) * BN_PAGE + pos % BN_PAGE) * a.vd;
-        for (int d = lane; d < a.vd; d += BN_WAVE) dst[d] = v[d];
+        if (a.v_transposed) {
+            T* dst = reinterpret_cast<T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * a.vd * BN_PAGE + pos % BN_PAGE;
+            for (int d = lane; d < a.vd; d += BN_WAVE) dst[(size_t)d * BN_PAGE] = v[d];
+        } else {
+            T* dst = reinterpret_cast<T*>(a.v_pages) + (((size_t)page * a.Hkv + kvh) * BN_PAGE + pos % BN_PAGE) * a.vd;
+            for (int d = lane; d < a.vd; d += BN_WAVE) dst[d] = v[d];
+        }
     }
 }
 
 extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positions, const int* seq_index,
                                 const int* block_table, int bt_stride, void* k_pages, void* v_pages, const float* wq,
                                 const float* wk, int n_tokens, int H, int Hkv, int hs, int vd, float eps, float temp_coef,
-                                int temp_every, hipStream_t s) {
+                                int temp_every, int v_transposed, hipStream_t s) {
     if (n_tokens <= 0 || H <= 0 || Hkv <= 0 || hs <= 0 || vd <= 0 || !qkv || !positions) return BN_ERR_ARG;
     if ((k_pages == nullptr) != (v_pages == nullptr) || (k_pages && (!seq_index || !block_table))) return BN_ERR_ARG;
     if ((wq == nullptr) != (wk == nullptr) || ld < H * hs + Hkv * (hs + vd)) return BN_ERR_ARG;
@@ -78,7 +85,7 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
     a.qkv = qkv; a.positions = positions; a.seq_index = seq_index; a.block_table = block_table;
     a.k_pages = k_pages; a.v_pages = v_pages; a.wq = wq; a.wk = wk;
     a.ld = ld; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv; a.hs = hs; a.vd = vd;
-    a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every;
+    a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every; a.v_transposed = v_transposed ? 1 : 0;
     const dim3 grid(n_tokens, H + 2 * Hkv);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, dim3(BN_WAVE), 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, dim3(BN_WAVE), 0, s, a);

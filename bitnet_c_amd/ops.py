@@ -52,7 +52,12 @@ _SIGNATURES = {
     },
     "qk_norm": {
         "bn_qk_norm_store": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
+                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_int, c_void_p],
+    },
+    "attn_mfma_general": {
+        "bn_attn_general_supports": [c_int, c_int],
+        "bn_attn_general_prompt": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
+                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p],
     },
     "state_mixers": {
         "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
@@ -936,6 +941,8 @@ def _check_pages(k_pages, v_pages, Hkv, hs, dtype, v_transposed=None, blocked=No
             raise KernelError(f"{nm}: expected contiguous [pages, {', '.join(map(str, shape))}], got {tuple(t.shape)}")
     if k_pages.shape[0] != v_pages.shape[0]:
         raise KernelError("k_pages and v_pages differ in their number of pages")
+    if k_pages.data_ptr() % 16 or v_pages.data_ptr() % 16:
+        raise KernelError("k_pages and v_pages must start at multiples of 16 bytes (the kernels load 16 bytes at a time)")
     return layout
 
 
@@ -1306,11 +1313,12 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
 
 def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *, v_dim: int = 0,
                   q_weight=None, k_weight=None, eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 0,
-                  seq_index=None, block_table=None, k_pages=None, v_pages=None) -> None:
+                  seq_index=None, block_table=None, k_pages=None, v_pages=None, v_transposed: bool = False) -> None:
     """In place on qkv [T, H hs + Hkv (hs + v_dim)]: every query and key head under an RMSNorm of its own (weights
     [hs] float32, shared by the heads; both or neither), the queries times 1 + temp_coef ln(floor((p + 1) / temp_every)
-    + 1) at position p (temp_every 0: no temperature); the normed keys and the values go into the pages (a row per
-    position) when pages are given.  Rows with position < 0 are left alone."""
+    + 1) at position p (temp_every 0: no temperature); the normed keys and the values go into the pages when pages are
+    given (keys a row per position; values the same way, or transposed inside a page when v_transposed).  Rows with
+    position < 0 are left alone."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
@@ -1324,7 +1332,7 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
             if w.numel() != hs or not w.is_contiguous():
                 raise KernelError(f"qk_norm_store: {nm} must hold {hs} float32 values")
     if k_pages is not None:
-        _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, False, False, vd)
+        _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, bool(v_transposed), False, vd)
         _dev(seq_index, "seq_index", torch.int32, 1)
         _dev(block_table, "block_table", torch.int32, 2)
         if seq_index.numel() != T or not block_table.is_contiguous():
@@ -1337,7 +1345,55 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         block_table.shape[1] if k_pages is not None else 0, k_pages.data_ptr() if k_pages is not None else None,
         v_pages.data_ptr() if k_pages is not None else None, q_weight.data_ptr() if q_weight is not None else None,
         k_weight.data_ptr() if k_weight is not None else None, T, H, Hkv, hs, vd, float(eps), float(temp_coef),
-        int(temp_every), _stream()), "qk_norm_store")
+        int(temp_every), int(bool(v_transposed)), _stream()), "qk_norm_store")
+
+
+GENERAL_PROMPT_TILE = 16       # query tokens of a tile of attention_general_prompt
+# BITNET_NO_GENERAL_MFMA=1 keeps the attention mixer's general form on the vector kernel in prompt steps too
+GENERAL_PROMPT_ON_MATRIX_CORES = os.environ.get("BITNET_NO_GENERAL_MFMA", "") in ("", "0")
+_GENERAL_SIZES = (32, 64, 96, 128, 256)
+
+
+def attention_general_supported(dtype, hs: int, v_dim: int) -> bool:
+    """Whether attention_general_prompt takes this type and these head sizes (bn_attn_general_supports, answered here so
+    that asking loads no kernel)."""
+    return dtype == torch.bfloat16 and int(hs) in _GENERAL_SIZES and int(v_dim) in _GENERAL_SIZES
+
+
+def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                             block_table: torch.Tensor, H: int, Hkv: int, hs: int, v_dim: int, scale: float, tiles: torch.Tensor,
+                             *, distance_bias=None, sink: bool = False) -> None:
+    """Causal prompt attention on the matrix cores for what attention() leaves to the vector kernel: bf16, keys 32, 64,
+    96, 128 or 256 wide, values of a width of their own from the same list, a distance bias and a sink (as attention()'s).
+    Pages: keys a row per position, values transposed.  tiles [n, 4] int32: (sequence, first row, rows <= 16, position of
+    the first), any order, tiles of no rows skipped.  out [T, H v_dim]."""
+    require_gpu()
+    _dev(qkv, "qkv", torch.bfloat16, 2)
+    _dev(out, "out", torch.bfloat16, 2)
+    if not attention_general_supported(qkv.dtype, hs, v_dim):
+        raise KernelError(f"attention_general_prompt: bf16 with head sizes from {_GENERAL_SIZES}, got {hs} and {v_dim}")
+    _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, True, False, v_dim)
+    _dev(block_table, "block_table", torch.int32, 2)
+    _dev(tiles, "tiles", torch.int32, 2)
+    T = qkv.shape[0]
+    if (H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * v_dim) or not out.is_contiguous() or tiles.shape[1] != 4
+            or not tiles.is_contiguous() or not block_table.is_contiguous()):
+        raise KernelError(f"attention_general_prompt: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} / tiles {tuple(tiles.shape)} "
+                          f"do not fit H={H} hs={hs} v_dim={v_dim}")
+    da = db = None
+    if distance_bias is not None:
+        da, db = distance_bias
+        for t, nm in ((da, "distance_bias[0]"), (db, "distance_bias[1]")):
+            _dev(t, nm, torch.float32, 1)
+            if t.numel() != H or not t.is_contiguous():
+                raise KernelError(f"attention_general_prompt: {nm} must hold one float32 per head")
+    if T == 0 or tiles.shape[0] == 0:
+        return
+    _check(_fn("attn_mfma_general", "bn_attn_general_prompt")(
+        qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * v_dim, k_pages.data_ptr(), v_pages.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], tiles.data_ptr(), tiles.shape[0], H, Hkv, hs, v_dim, float(scale),
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), _stream()),
+        "attention_general_prompt")
 
 
 # --------------------------------------------------------------------------------------

@@ -105,8 +105,9 @@ class Attention(Part):
         return [self.qkv, self.o]
 
     def cache_need(self) -> CacheNeed:
-        if self.general:                  # the vector kernel's pages, in both types
-            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_head_dim=self.vd, v_layout="rows"))
+        if self.general:                  # keys a row per position, values transposed inside a page, in both types: what the
+            # vector kernel and the general prompt kernel on the matrix cores both read
+            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_head_dim=self.vd, v_layout="transposed"))
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 
     def wants_deferred_norm(self, ctx, rows: int) -> bool:
@@ -133,7 +134,8 @@ class Attention(Part):
         ops.qk_norm_store(qkv, ctx.positions, H, Hkv, hs, v_dim=vd, q_weight=self.q_norm, k_weight=self.k_norm,
                           eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
                           seq_index=ctx.seq_index if kv.writes else None, block_table=kv.block_table if kv.writes else None,
-                          k_pages=kv.k_pages if kv.writes else None, v_pages=kv.v_pages if kv.writes else None)
+                          k_pages=kv.k_pages if kv.writes else None, v_pages=kv.v_pages if kv.writes else None,
+                          v_transposed=True)
         out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
         bias = (self.dist_a, self.dist_b) if self.distance_bias else None
         if ctx.is_decode:
@@ -141,12 +143,15 @@ class Attention(Part):
                                                                            target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=False, blocked=False,
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=True, blocked=False,
                           v_dim=vd, distance_bias=bias, sink=self.sink)
+        elif not self.window and ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES:
+            ops.attention_general_prompt(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, vd, self.scale,
+                                         ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self.sink)
         else:
             _, _, qt = ops.attention_row_shape(H, Hkv, False)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
-                          tiles=ctx.tiles(qt), qt=qt, v_transposed=False, blocked=False, v_dim=vd, distance_bias=bias,
+                          tiles=ctx.tiles(qt), qt=qt, v_transposed=True, blocked=False, v_dim=vd, distance_bias=bias,
                           sink=self.sink)
         return self.o(out)
 

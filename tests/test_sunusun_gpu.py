@@ -193,7 +193,7 @@ def test_mingru_alone(dtype, W):
     assert bool((state[0] == 0).all())
 
 
-def _attention_case(dtype, H, G, hs, vd, lens, seed, scale=0.4, spike=None):
+def _attention_case(dtype, H, G, hs, vd, lens, seed, scale=0.4, spike=None, transposed=False):
     """Random q, k, v for one sequence; returns what the kernels give for the whole prompt and the plain result.
     spike = (query position, key position): that pair's score is made to stand out."""
     from bitnet_c_amd import ops
@@ -225,7 +225,7 @@ def _attention_case(dtype, H, G, hs, vd, lens, seed, scale=0.4, spike=None):
     want = want.reshape(T, H * vd)
     n_pages = -(-T // PAGE)
     kp = torch.zeros(n_pages + 3, G, PAGE, hs, dtype=dtype, device=dev)
-    vp = torch.zeros(n_pages + 3, G, PAGE, vd, dtype=dtype, device=dev)
+    vp = torch.zeros((n_pages + 3, G, vd, PAGE) if transposed else (n_pages + 3, G, PAGE, vd), dtype=dtype, device=dev)
     table = (torch.randperm(n_pages + 3, generator=g)[:n_pages]).to(torch.int32).view(1, -1).to(dev).contiguous()
     args = dict(q_weight=wq.to(dev), k_weight=wk.to(dev), eps=eps, temp_coef=coef, temp_every=every)
     return dict(qkv=qkv, want=want, kp=kp, vp=vp, table=table, args=args, bias=(da.to(dev), db.to(dev)), scale=scale)
@@ -264,6 +264,61 @@ def test_attention_pieces_alone(dtype, H, G, hs, vd):
                       chunk=chunk, v_transposed=False, blocked=False, v_dim=vd, distance_bias=c["bias"], sink=True)
         outs.append(out)
     close(torch.cat(outs), c["want"], dtype)
+
+
+@pytest.mark.parametrize("H,G,hs,vd", [(4, 2, 64, 64), (2, 1, 128, 32), (3, 3, 32, 96), (5, 1, 96, 128), (2, 2, 256, 256)])
+def test_general_prompt_attention_on_the_matrix_cores(H, G, hs, vd):
+    """The bf16 prompt kernel for the same mixer (keys a row per position, values transposed): a prompt in two portions
+    whose tiles end in partial ones, the second portion reading the first's pages, and the tokens decoded behind it by the
+    vector kernel over the same pages."""
+    from bitnet_c_amd import ops
+    dev, T, dtype = "cuda:0", 181, torch.bfloat16
+    c = _attention_case(dtype, H, G, hs, vd, T, seed=H * 1000 + hs + vd, scale=1.0 / math.sqrt(hs), transposed=True)
+    outs = []
+    for lo, hi in ((0, 70), (70, 150)):
+        n = hi - lo
+        rows = c["qkv"][lo:hi].to(dev).contiguous()
+        pos = torch.arange(lo, hi, dtype=torch.int32, device=dev)
+        ops.qk_norm_store(rows, pos, H, G, hs, v_dim=vd, seq_index=torch.zeros(n, dtype=torch.int32, device=dev),
+                          block_table=c["table"], k_pages=c["kp"], v_pages=c["vp"], v_transposed=True, **c["args"])
+        qt = ops.GENERAL_PROMPT_TILE
+        tiles = [[0, i, min(qt, n - i), lo + i] for i in range(0, n, qt)] + [[0, 0, 0, 0]]        # and a tile of no rows
+        tiles = torch.tensor(tiles[::-1], dtype=torch.int32, device=dev)                          # in any order
+        out = torch.full((n, H * vd), 7.0, dtype=dtype, device=dev)
+        ops.attention_general_prompt(rows, out, c["kp"], c["vp"], c["table"], H, G, hs, vd, c["scale"], tiles,
+                                     distance_bias=c["bias"], sink=True)
+        outs.append(out)
+    for t in range(150, T):
+        rows = c["qkv"][t:t + 1].to(dev).contiguous()
+        pos = torch.tensor([t], dtype=torch.int32, device=dev)
+        ops.qk_norm_store(rows, pos, H, G, hs, v_dim=vd, seq_index=torch.zeros(1, dtype=torch.int32, device=dev),
+                          block_table=c["table"], k_pages=c["kp"], v_pages=c["vp"], v_transposed=True, **c["args"])
+        out = torch.empty(1, H * vd, dtype=dtype, device=dev)
+        ops.attention(rows, out, c["kp"], c["vp"], c["table"], H, G, hs, c["scale"], seq_lens=pos + 1, v_transposed=True,
+                      blocked=False, v_dim=vd, distance_bias=c["bias"], sink=True)
+        outs.append(out)
+    close(torch.cat(outs), c["want"], dtype)
+
+
+@pytest.mark.parametrize("key", [0, 1, 31, 32, 63, 64, 65, 2047, 2048, 2100])
+def test_a_far_key_on_the_matrix_cores(key):
+    """One key whose score stands out, at the first positions and at the borders of the kernel's blocks of 32 keys and of
+    the pages, seen from the last tokens of a prompt of 2,113 tokens, with and without the sink."""
+    from bitnet_c_amd import ops
+    dev, H, G, hs, vd, T, dtype = "cuda:0", 2, 1, 32, 32, 2113, torch.bfloat16
+    c = _attention_case(dtype, H, G, hs, vd, T, seed=key, scale=1.5, spike=(T - 1, key), transposed=True)
+    rows = c["qkv"].to(dev).contiguous()
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    ops.qk_norm_store(rows, pos, H, G, hs, v_dim=vd, seq_index=torch.zeros(T, dtype=torch.int32, device=dev),
+                      block_table=c["table"], k_pages=c["kp"], v_pages=c["vp"], v_transposed=True, **c["args"])
+    qt = ops.GENERAL_PROMPT_TILE
+    tiles = torch.tensor([[0, i, min(qt, T - i), i] for i in range(0, T, qt)], dtype=torch.int32, device=dev)
+    out = torch.empty(T, H * vd, dtype=dtype, device=dev)
+    ops.attention_general_prompt(rows, out, c["kp"], c["vp"], c["table"], H, G, hs, vd, c["scale"], tiles,
+                                 distance_bias=c["bias"], sink=True)
+    close(out[-40:], c["want"][-40:], dtype, bf16_rows=0.05)
+    close(out[:70], c["want"][:70], dtype, bf16_rows=0.05)
+    assert float(out[-1].float().abs().max()) > 2.0              # the key's value (shifted by 5) dominates
 
 
 def test_the_sink_alone_takes_weight_when_every_score_is_low():

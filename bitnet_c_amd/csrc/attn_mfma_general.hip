@@ -70,17 +70,31 @@ __global__ __launch_bounds__(AG_WAVES * BN_WAVE) void attn_general_prompt_kernel
     const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
     const int krow = 8 * (i >> 2) + (i & 3);             // this lane's key row of tile 0 inside a block; tile 1: 4 further
 
+    // The keys of a block are asked for one block ahead (the last block asks for itself once more: a load without a
+    // branch around it), so that the first product finds its operand there; the values are asked for when the block
+    // begins and are used behind the weights.
+    bf16x8 kn0[DC], kn1[DC];
+    auto ask_keys = [&](int kb) {
+        const int page = a.block_table[(size_t)seq * a.bt_stride + kb / BN_PAGE];
+        const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + kb % BN_PAGE + krow) * HS + 8 * g;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) { kn0[c] = ag_ld16(kbase + 32 * c); kn1[c] = ag_ld16(kbase + 4 * HS + 32 * c); }
+    };
+    ask_keys(0);
+    const int last_block = ((k_hi - 1) / 32) * 32;
     for (int kb = 0; kb < k_hi; kb += 32) {
         const int page = a.block_table[(size_t)seq * a.bt_stride + kb / BN_PAGE];
         const int off = kb % BN_PAGE;
-        const bf16* kbase = a.k_pages + (((size_t)page * a.Hkv + kvh) * BN_PAGE + off + krow) * HS + 8 * g;
         const bf16* vbase = a.v_pages + (((size_t)page * a.Hkv + kvh) * VD + i) * BN_PAGE + off + 8 * g;
+        bf16x8 k0[DC], k1[DC];
+#pragma unroll
+        for (int c = 0; c < DC; ++c) { k0[c] = kn0[c]; k1[c] = kn1[c]; }
+        ask_keys(min(kb + 32, last_block));
         f32x4 st0 = (f32x4){0.f, 0.f, 0.f, 0.f}, st1 = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
-            const bf16x8 k0 = ag_ld16(kbase + 32 * c), k1 = ag_ld16(kbase + 4 * HS + 32 * c);
-            st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[c], st0, 0, 0, 0);
-            st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[c], st1, 0, 0, 0);
+            st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0[c], qf[c], st0, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1[c], qf[c], st1, 0, 0, 0);
         }
         // the values' tiles are asked for now and used behind the weights
         bf16x8 va[DT];

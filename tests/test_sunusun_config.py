@@ -63,7 +63,7 @@ def test_cache_needs_a_state_per_entry_and_pages_per_attention():
                 rows *= 2                          # the kernel holds a head's rows rounded up to a power of two times 16
             assert need.kv is None and need.state.shape == (m["heads"] * rows * m["dim"] + raw["width"],)
         else:
-            assert need.state.shape == (m["right"]["width"],) and need.kv.v_layout == "rows"
+            assert need.state.shape == (m["right"]["width"],) and need.kv.v_layout == "transposed"
             assert (need.kv.n_kv_heads, need.kv.head_dim, need.kv.v_dim) == (m["left"]["kv_heads"], m["left"]["dim"], m["left"]["vdim"])
         assert need.state.device_addressed and need.state.dtype == torch.float32
     cache = PagedCache(needs, [None] * len(needs), 256, dtype=torch.float32, device=None)

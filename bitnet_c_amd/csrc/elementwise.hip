@@ -625,3 +625,60 @@ extern "C" int bn_rmsnorm_mean(int dtype, void* out, const void* a, const void* 
         return BN_ERR_DTYPE;
     return bn_launch_status();
 }
+
+// A part's output that has a norm of its own before it joins the stream, and the norm of the next part, in one pass over
+// the row:   x += wb * d / sqrt(mean(d^2) + eps_b),   out = w * x / sqrt(mean(x^2) + eps)   (out and w null: the sum alone).
+// d is the sum of n_parts slabs (part_stride elements apart, added in slab order) of type TD.  Everything in float32; the
+// row of d is formed once and kept in shared memory (dim floats) between the two passes.
+template <typename T, typename TD>
+__global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_parts, size_t part_stride,
+                                          const float* __restrict__ wb, float eps_b, const float* __restrict__ w,
+                                          T* __restrict__ out, int dim, float eps) {
+    extern __shared__ float row[];
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    float* xr = x + (size_t)r * dim;
+    const TD* dr = delta + (size_t)r * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        float d = 0.f;
+        for (int p = 0; p < n_parts; ++p) d += to_f32(dr[p * part_stride + i]);
+        row[i] = d;
+        ss = fmaf(d, d, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float fb = 1.0f / sqrtf(ss / (float)dim + eps_b);
+    float sx = 0.f;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+        const float v = xr[i] + row[i] * fb * wb[i];
+        xr[i] = v;
+        row[i] = v;
+        sx = fmaf(v, v, sx);
+    }
+    if (!out) return;
+    sx = block_sum(sx, scratch);
+    const float f = 1.0f / sqrtf(sx / (float)dim + eps);
+    T* o = out + (size_t)r * dim;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_f32<T>(row[i] * f * w[i]);
+}
+
+// dtype: the type of out (and of delta when parts_f32 is 0); parts_f32: delta is n_parts float32 slabs [n_parts][n_rows][dim]
+extern "C" int bn_add_normed_rmsnorm(int dtype, void* x, const void* delta, int n_parts, int parts_f32, const float* wb,
+                                     float eps_b, const float* w, void* out, int n_rows, int dim, float eps, hipStream_t s) {
+    if (n_rows <= 0 || dim <= 0 || dim > 16384 || n_parts < 1 || !x || !delta || !wb || ((w == nullptr) != (out == nullptr)))
+        return BN_ERR_ARG;
+    if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
+    const int threads = dim >= 2048 ? 512 : 256;
+    const size_t shm = (size_t)dim * sizeof(float), stride = (size_t)n_rows * dim;
+    const dim3 grid(n_rows), block(threads);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL((add_normed_rmsnorm_kernel<float, float>), grid, block, shm, s, (float*)x, (const float*)delta, n_parts,
+                           stride, wb, eps_b, w, (float*)out, dim, eps);
+    else if (parts_f32)
+        hipLaunchKernelGGL((add_normed_rmsnorm_kernel<bf16, float>), grid, block, shm, s, (float*)x, (const float*)delta, n_parts,
+                           stride, wb, eps_b, w, (bf16*)out, dim, eps);
+    else
+        hipLaunchKernelGGL((add_normed_rmsnorm_kernel<bf16, bf16>), grid, block, shm, s, (float*)x, (const bf16*)delta, n_parts,
+                           stride, wb, eps_b, w, (bf16*)out, dim, eps);
+    return bn_launch_status();
+}

@@ -1,0 +1,143 @@
+// Kernels of the latent attention mixer: keys and values are both projections of one normed vector c per token (the
+// latent), which is all that the cache keeps.  Because k_h = U_h c and v_h = V_h c are linear in c, the mixer attends in
+// the latent's space: the query of head h becomes q'_h = U_h^T q_h, all heads share the one cached vector as key and as
+// value (score = q'_h . c, o'_h = sum_j p_j c_j), and the value projection runs once on the result, o_h = V_h o'_h.
+//
+//   bn_latent_store   c = x / sqrt(mean(x^2) + eps) * w over the latent's columns of a projected row -> the page of the
+//                     row's position, once as a key row and once into the transposed value page
+//   bn_head_linear    y[t, h, :] = x[t, h, :] . M_h for every head (M_h [in, out]), optionally times sigmoid(gate[t, h, :])
+//   bn_sigmoid_gate   y *= sigmoid(gate), element by element
+// All arithmetic in float32; results are stored once in the activations' type.
+#include "common.h"
+#include <math.h>
+
+struct LatentStoreArgs {
+    const void* x;            // [T, ld]; the latent's columns start at column `col`
+    const int* positions;     // [T]; < 0: a padding row, nothing is written
+    const int* seq_index;     // [T] row of the block table
+    const int* block_table;   // [n_seqs, bt_stride]
+    void* k_pages;            // [pages, 1, BN_PAGE, rank]
+    void* v_pages;            // [pages, 1, rank, BN_PAGE]
+    const float* w;           // [rank]
+    int ld, col, rank, bt_stride;
+    float eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_store_kernel(LatentStoreArgs a) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const int pos = a.positions[t];
+    if (pos < 0) return;
+    const T* x = reinterpret_cast<const T*>(a.x) + (size_t)t * a.ld + a.col;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < a.rank; d += blockDim.x) { const float v = to_f32(x[d]); ss = fmaf(v, v, ss); }
+    ss = block_sum(ss, scratch);
+    const float f = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
+    const int page = a.block_table[(size_t)a.seq_index[t] * a.bt_stride + pos / BN_PAGE], slot = pos % BN_PAGE;
+    T* kd = reinterpret_cast<T*>(a.k_pages) + ((size_t)page * BN_PAGE + slot) * a.rank;
+    T* vd = reinterpret_cast<T*>(a.v_pages) + (size_t)page * a.rank * BN_PAGE + slot;
+    for (int d = threadIdx.x; d < a.rank; d += blockDim.x) {
+        const T c = from_f32<T>(to_f32(x[d]) * f * a.w[d]);
+        kd[d] = c;
+        vd[(size_t)d * BN_PAGE] = c;
+    }
+}
+
+extern "C" int bn_latent_store(int dtype, const void* x, int ld, int col, const int* positions, const int* seq_index,
+                               const int* block_table, int bt_stride, void* k_pages, void* v_pages, const float* w, int n_tokens,
+                               int rank, float eps, hipStream_t s) {
+    if (n_tokens <= 0 || rank <= 0 || col < 0 || ld < col + rank) return BN_ERR_ARG;
+    if (!x || !positions || !seq_index || !block_table || !k_pages || !v_pages || !w) return BN_ERR_ARG;
+    LatentStoreArgs a;
+    a.x = x; a.positions = positions; a.seq_index = seq_index; a.block_table = block_table; a.k_pages = k_pages;
+    a.v_pages = v_pages; a.w = w; a.ld = ld; a.col = col; a.rank = rank; a.bt_stride = bt_stride; a.eps = eps;
+    const dim3 grid(n_tokens), block(rank > 128 ? 256 : 64);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(latent_store_kernel<float>, grid, block, 0, s, a);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(latent_store_kernel<bf16>, grid, block, 0, s, a);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- a product per head ---------------------------------------------------------------------------------------------
+#define HL_ROWS 8             // rows of x that a workgroup takes
+#define HL_COLS 128           // output columns of a workgroup: one a thread
+
+struct HeadLinearArgs {
+    const void* x;            // [T, ldx]: head h at h * I
+    const void* w;            // [H, I, O]
+    void* y;                  // [T, ldy]: head h at h * O
+    const void* gate;         // [T, ldg]: head h at h * O; null: none
+    int ldx, ldy, ldg, T, H, I, O;
+};
+
+// The rows of x are staged in shared memory as float32 and read by every thread at the same address; a thread walks the
+// input dimension with one coalesced load of the weights a step.
+template <typename T>
+__global__ __launch_bounds__(HL_COLS) void head_linear_kernel(HeadLinearArgs a) {
+    extern __shared__ float xs[];                        // [HL_ROWS][I]
+    const int h = blockIdx.y, t0 = blockIdx.z * HL_ROWS, o = blockIdx.x * HL_COLS + threadIdx.x;
+    const int rows = min(HL_ROWS, a.T - t0);
+    const T* x = reinterpret_cast<const T*>(a.x);
+    for (int idx = threadIdx.x; idx < HL_ROWS * a.I; idx += HL_COLS) {
+        const int r = idx / a.I, i = idx - r * a.I;
+        xs[idx] = r < rows ? to_f32(x[(size_t)(t0 + r) * a.ldx + (size_t)h * a.I + i]) : 0.f;
+    }
+    __syncthreads();
+    if (o >= a.O) return;
+    float acc[HL_ROWS];
+#pragma unroll
+    for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
+    const T* w = reinterpret_cast<const T*>(a.w) + (size_t)h * a.I * a.O + o;
+    for (int i = 0; i < a.I; ++i) {
+        const float wv = to_f32(w[(size_t)i * a.O]);
+#pragma unroll
+        for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(xs[r * a.I + i], wv, acc[r]);
+    }
+    T* y = reinterpret_cast<T*>(a.y);
+    const T* g = reinterpret_cast<const T*>(a.gate);
+#pragma unroll
+    for (int r = 0; r < HL_ROWS; ++r) {
+        if (r >= rows) break;
+        float v = acc[r];
+        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + (size_t)h * a.O + o])));
+        y[(size_t)(t0 + r) * a.ldy + (size_t)h * a.O + o] = from_f32<T>(v);
+    }
+}
+
+extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, void* y, int ldy, const void* gate, int ldg,
+                              int n_rows, int H, int I, int O, hipStream_t s) {
+    if (n_rows <= 0 || H <= 0 || I <= 0 || O <= 0 || !x || !w || !y) return BN_ERR_ARG;
+    if (ldx < H * I || ldy < H * O || (gate && ldg < H * O) || (size_t)HL_ROWS * I * sizeof(float) > 64 * 1024 || H > 65535) return BN_ERR_ARG;
+    const int row_tiles = (n_rows + HL_ROWS - 1) / HL_ROWS;
+    if (row_tiles > 65535) return BN_ERR_ARG;
+    HeadLinearArgs a;
+    a.x = x; a.w = w; a.y = y; a.gate = gate; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.T = n_rows; a.H = H; a.I = I; a.O = O;
+    const dim3 grid((O + HL_COLS - 1) / HL_COLS, H, row_tiles), block(HL_COLS);
+    const size_t shm = (size_t)HL_ROWS * I * sizeof(float);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(head_linear_kernel<float>, grid, block, shm, s, a);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(head_linear_kernel<bf16>, grid, block, shm, s, a);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- y *= sigmoid(gate) ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, int ldy, const T* __restrict__ g, int ldg, int n_rows, int n_cols) {
+    const size_t n = (size_t)n_rows * n_cols;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = idx / n_cols, c = idx - r * n_cols;
+        const float v = to_f32(y[r * ldy + c]) / (1.0f + expf(-to_f32(g[r * ldg + c])));
+        y[r * ldy + c] = from_f32<T>(v);
+    }
+}
+
+extern "C" int bn_sigmoid_gate(int dtype, void* y, int ldy, const void* gate, int ldg, int n_rows, int n_cols, hipStream_t s) {
+    if (n_rows <= 0 || n_cols <= 0 || ldy < n_cols || ldg < n_cols || !y || !gate) return BN_ERR_ARG;
+    const size_t n = (size_t)n_rows * n_cols;
+    const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)y, ldy, (const float*)gate, ldg, n_rows, n_cols);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(sigmoid_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)y, ldy, (const bf16*)gate, ldg, n_rows, n_cols);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}

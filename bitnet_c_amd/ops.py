@@ -49,10 +49,26 @@ _SIGNATURES = {
         "bn_unary_act_apply": [c_int, c_void_p, c_void_p, c_longlong, c_int, c_void_p],
         "bn_scale": [c_void_p, c_longlong, c_float, c_void_p],
         "bn_rmsnorm_mean": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
+        "bn_add_normed_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int,
+                                  c_float, c_void_p],
     },
     "qk_norm": {
         "bn_qk_norm_store": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_int, c_void_p],
+                             c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_int, c_int, c_void_p, c_int,
+                             c_int, c_void_p],
+    },
+    "latent": {
+        "bn_latent_store": [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                            c_int, c_int, c_float, c_void_p],
+        "bn_head_linear": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p],
+        "bn_sigmoid_gate": [c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    },
+    "moe": {
+        "bn_moe_route": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_void_p],
+        "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                           c_int, c_int, c_void_p],
     },
     "attn_mfma_general": {
         "bn_attn_general_supports": [c_int, c_int],
@@ -1313,12 +1329,16 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
 
 def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *, v_dim: int = 0,
                   q_weight=None, k_weight=None, eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 0,
-                  seq_index=None, block_table=None, k_pages=None, v_pages=None, v_transposed: bool = False) -> None:
+                  seq_index=None, block_table=None, k_pages=None, v_pages=None, v_transposed: bool = False,
+                  norm_projection: bool = False, inv_freq=None, rope_dims: int = 0, rope_interleaved: bool = False) -> None:
     """In place on qkv [T, H hs + Hkv (hs + v_dim)]: every query and key head under an RMSNorm of its own (weights
-    [hs] float32, shared by the heads; both or neither), the queries times 1 + temp_coef ln(floor((p + 1) / temp_every)
-    + 1) at position p (temp_every 0: no temperature); the normed keys and the values go into the pages when pages are
-    given (keys a row per position; values the same way, or transposed inside a page when v_transposed).  Rows with
-    position < 0 are left alone."""
+    [hs] float32, shared by the heads; both or neither), or, with norm_projection, one RMSNorm over the whole query
+    projection and one over the whole key projection (weights [H hs] and [Hkv hs]); then the first rope_dims dimensions
+    of every query and key head rotated by the position (inv_freq [rope_dims / 2] float32; pairs (2i, 2i + 1) when
+    rope_interleaved, (i, i + rope_dims / 2) otherwise; inv_freq None: no rotation); the queries times
+    1 + temp_coef ln(floor((p + 1) / temp_every) + 1) at position p (temp_every 0: no temperature); the keys and the
+    values go into the pages when pages are given (keys a row per position; values the same way, or transposed inside a
+    page when v_transposed).  Rows with position < 0 are left alone."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
@@ -1326,11 +1346,18 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
     T = qkv.shape[0]
     if positions.numel() != T or qkv.shape[1] < H * hs + Hkv * (hs + vd) or (q_weight is None) != (k_weight is None):
         raise KernelError(f"qk_norm_store: qkv {tuple(qkv.shape)} does not fit H={H} Hkv={Hkv} hs={hs} v_dim={vd}")
-    for w, nm in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+    for w, nm, heads in ((q_weight, "q_weight", H), (k_weight, "k_weight", Hkv)):
         if w is not None:
             _dev(w, nm, torch.float32, 1)
-            if w.numel() != hs or not w.is_contiguous():
-                raise KernelError(f"qk_norm_store: {nm} must hold {hs} float32 values")
+            want = hs * heads if norm_projection else hs
+            if w.numel() != want or not w.is_contiguous():
+                raise KernelError(f"qk_norm_store: {nm} must hold {want} float32 values")
+    if hs > MAX_HEAD_DIM:
+        raise KernelError(f"qk_norm_store: head size {hs} is above {MAX_HEAD_DIM}")
+    if inv_freq is not None:
+        _dev(inv_freq, "inv_freq", torch.float32, 1)
+        if rope_dims <= 0 or rope_dims % 2 or rope_dims > hs or inv_freq.numel() != rope_dims // 2 or not inv_freq.is_contiguous():
+            raise KernelError(f"qk_norm_store: rope_dims {rope_dims} does not fit hs={hs} / inv_freq {tuple(inv_freq.shape)}")
     if k_pages is not None:
         _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, bool(v_transposed), False, vd)
         _dev(seq_index, "seq_index", torch.int32, 1)
@@ -1345,7 +1372,9 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         block_table.shape[1] if k_pages is not None else 0, k_pages.data_ptr() if k_pages is not None else None,
         v_pages.data_ptr() if k_pages is not None else None, q_weight.data_ptr() if q_weight is not None else None,
         k_weight.data_ptr() if k_weight is not None else None, T, H, Hkv, hs, vd, float(eps), float(temp_coef),
-        int(temp_every), int(bool(v_transposed)), _stream()), "qk_norm_store")
+        int(temp_every), int(bool(v_transposed)), int(bool(norm_projection)),
+        inv_freq.data_ptr() if inv_freq is not None else None, int(rope_dims), int(bool(rope_interleaved)), _stream()),
+        "qk_norm_store")
 
 
 GENERAL_PROMPT_TILE = 16       # query tokens of a tile of attention_general_prompt
@@ -1628,6 +1657,179 @@ def mingru_scan(zxg: torch.Tensor, bias_z, bias_x, state: torch.Tensor, slot_ids
             bias_z.data_ptr() if bias_z is not None else None, bias_x.data_ptr() if bias_x is not None else None,
             state.data_ptr(), stride, tl, n_tiles, sl, slot_ids.data_ptr(), W, _stream()), "mingru_scan")
     return y
+
+
+# --------------------------------------------------------------------------------------
+# a part's output with a norm of its own; latent attention; mixture of experts
+# --------------------------------------------------------------------------------------
+
+def add_normed_rmsnorm(x: torch.Tensor, delta, out_weight: torch.Tensor, out_eps: float, weight: Optional[torch.Tensor] = None,
+                       eps: float = 0.0, out_dtype=None):
+    """x (float32, [T, D]) += out_weight * delta / sqrt(mean(delta^2) + out_eps), row by row in float32; delta [T, D]
+    in x's or the activations' type, or PartialSums (its slabs are added first).  With `weight`, also returns the rows of
+    the new x under an RMSNorm (weight, eps) in out_dtype: a block's output norm, the residual sum and the next part's
+    norm in one kernel."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    _dev(out_weight, "out_weight", torch.float32, 1)
+    T, D = x.shape
+    parts = delta if isinstance(delta, PartialSums) else None
+    d = parts.slabs if parts is not None else delta
+    _dev(d, "delta")
+    if tuple(parts.shape if parts is not None else d.shape) != (T, D) or not d.is_contiguous() or not x.is_contiguous():
+        raise KernelError(f"add_normed_rmsnorm: delta does not match x {tuple(x.shape)}, or is not contiguous")
+    if out_weight.numel() != D or not out_weight.is_contiguous() or D > 16384:
+        raise KernelError(f"add_normed_rmsnorm: the output norm's weight must hold {D} (at most 16,384) values")
+    if parts is None and d.dtype not in _DT:
+        raise KernelError(f"add_normed_rmsnorm: unsupported delta type {d.dtype}")
+    out = None
+    if weight is not None:
+        _dev(weight, "weight", torch.float32, 1)
+        if weight.numel() != D or not weight.is_contiguous():
+            raise KernelError(f"add_normed_rmsnorm: weight must hold {D} values")
+        out = torch.empty((T, D), dtype=out_dtype or (torch.float32 if parts is not None else d.dtype), device=x.device)
+    # the kernel's type names the type of out and of a delta that is no float32 slab
+    code = _code(out.dtype) if out is not None else (_code(torch.float32) if parts is not None else _code(d.dtype))
+    if parts is None and out is not None and out.dtype != d.dtype:
+        raise KernelError("add_normed_rmsnorm: delta and the normed rows have one type")
+    if T == 0:
+        return out
+    _check(_fn("elementwise", "bn_add_normed_rmsnorm")(
+        code, x.data_ptr(), d.data_ptr(), parts.slabs.shape[0] if parts is not None else 1, int(parts is not None),
+        out_weight.data_ptr(), float(out_eps), weight.data_ptr() if weight is not None else None,
+        out.data_ptr() if out is not None else None, T, D, float(eps), _stream()), "add_normed_rmsnorm")
+    return out
+
+
+def latent_store(x: torch.Tensor, col: int, rank: int, weight: torch.Tensor, eps: float, positions, seq_index, block_table,
+                 k_pages: torch.Tensor, v_pages: torch.Tensor) -> None:
+    """Columns col .. col + rank of every row of x under an RMSNorm (weight [rank] float32, eps inside the root, float32
+    arithmetic), stored at the row's position of its sequence's pages: as a key row ([pages, 1, PAGE, rank]) and into the
+    transposed value page ([pages, 1, rank, PAGE]).  Rows with position < 0 store nothing."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(weight, "weight", torch.float32, 1)
+    _dev(positions, "positions", torch.int32, 1)
+    _dev(seq_index, "seq_index", torch.int32, 1)
+    _dev(block_table, "block_table", torch.int32, 2)
+    T = x.shape[0]
+    _check_pages(k_pages, v_pages, 1, rank, x.dtype, True, False, rank)
+    if (col < 0 or x.shape[1] < col + rank or weight.numel() != rank or not weight.is_contiguous() or positions.numel() != T
+            or seq_index.numel() != T or not block_table.is_contiguous()):
+        raise KernelError(f"latent_store: x {tuple(x.shape)} / columns {col}..{col + rank} / weight {tuple(weight.shape)} do not fit")
+    if T == 0:
+        return
+    _check(_fn("latent", "bn_latent_store")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), int(col), positions.data_ptr(),
+                                            seq_index.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+                                            k_pages.data_ptr(), v_pages.data_ptr(), weight.data_ptr(), T, int(rank), float(eps),
+                                            _stream()), "latent_store")
+
+
+HEAD_LINEAR_MAX_IN = 2048          # the kernel stages 8 rows of a head's input as float32 in 64 KB of shared memory
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] = None, *,
+                allow_library: Optional[bool] = None) -> torch.Tensor:
+    """A product per head: y[t, h, :] = x[t, h, :] . w[h] with x [T, H I] (rows contiguous), w [H, I, O] -> y [T, H O];
+    with `gate` [T, H O] (rows contiguous) y is multiplied by sigmoid(gate) element by element.  float32 accumulation.
+    bf16 with more than SKINNY_ROWS rows goes to the library's batched product (allow_library as linear's), everything else
+    to a kernel that reads every head's matrix once for 8 rows."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(w, "w", x.dtype, 3)
+    T = x.shape[0]
+    H, I, O = w.shape
+    if x.shape[1] != H * I or not w.is_contiguous():
+        raise KernelError(f"head_linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    if gate is not None:
+        _dev(gate, "gate", x.dtype, 2)
+        if tuple(gate.shape) != (T, H * O):
+            raise KernelError(f"head_linear: gate {tuple(gate.shape)} is not [{T}, {H * O}]")
+    y = torch.empty((T, H * O), dtype=x.dtype, device=x.device)
+    if T == 0:
+        return y
+    if allow_library is None:
+        allow_library = LIBRARY_PRODUCTS
+    ldx = _rows(x, "x")
+    if x.dtype == torch.bfloat16 and T > SKINNY_ROWS and allow_library:
+        xv = x.as_strided((H, T, I), (I, ldx, 1))
+        torch.bmm(xv, w, out=y.view(T, H, O).transpose(0, 1))
+        if gate is not None:
+            _check(_fn("latent", "bn_sigmoid_gate")(_code(y.dtype), y.data_ptr(), H * O, gate.data_ptr(), _rows(gate, "gate"),
+                                                    T, H * O, _stream()), "sigmoid_gate")
+        return y
+    if I > HEAD_LINEAR_MAX_IN:
+        raise KernelError(f"head_linear: a head's input of {I} values is above {HEAD_LINEAR_MAX_IN}")
+    _check(_fn("latent", "bn_head_linear")(_code(x.dtype), x.data_ptr(), ldx, w.data_ptr(), y.data_ptr(), H * O,
+                                           gate.data_ptr() if gate is not None else None,
+                                           _rows(gate, "gate") if gate is not None else 0, T, H, I, O, _stream()), "head_linear")
+    return y
+
+
+MOE_MAX_EXPERTS = _build.header_constant("MOE_MAX_EXPERTS", "moe.hip")
+MOE_SCORINGS = {"sigmoid": _build.header_constant("MOE_SCORE_SIGMOID", "moe.hip"),
+                "softmax": _build.header_constant("MOE_SCORE_SOFTMAX", "moe.hip")}
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = "sigmoid", renormalize: bool = False):
+    """(ids [T, top_k] int32, weights [T, top_k] float32): router logits z = router . h in float32 (router [E, D]
+    float32, h in the activations' type), scores sigmoid(z) or softmax(z) over the experts, the top_k largest in
+    descending order (ties: the lower index); renormalize divides the chosen scores by their sum."""
+    require_gpu()
+    _dev(h, "h", dims=2)
+    _dev(router, "router", torch.float32, 2)
+    T, D = h.shape
+    E = router.shape[0]
+    if scoring not in MOE_SCORINGS:
+        raise KernelError(f"moe_route: unknown scoring {scoring!r}; known: {sorted(MOE_SCORINGS)}")
+    if router.shape[1] != D or not router.is_contiguous() or not 1 <= top_k <= E or E > MOE_MAX_EXPERTS or D > 16384:
+        raise KernelError(f"moe_route: h {tuple(h.shape)}, router {tuple(router.shape)}, top_k {top_k} do not fit "
+                          f"(at most {MOE_MAX_EXPERTS} experts, 16,384 columns)")
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top_k), dtype=torch.float32, device=h.device)
+    if T:
+        _check(_fn("moe", "bn_moe_route")(_code(h.dtype), h.data_ptr(), _rows(h, "h"), router.data_ptr(), ids.data_ptr(),
+                                          wts.data_ptr(), T, D, E, int(top_k), MOE_SCORINGS[scoring], int(bool(renormalize)),
+                                          _stream()), "moe_route")
+    return ids, wts
+
+
+def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
+                activation: str = "relu2", weight_on_input: bool = True) -> PartialSums:
+    """The chosen experts' outputs, expert e being w_down[e] act(w_up[e] x) (w_up [E, F, D], w_down [E, D, F], act one of
+    UNARY_ACTIVATIONS): slab j of the result [top_k, T, D] (float32) holds every token's j-th choice, computed on w h
+    (weight_on_input) or scaled by w afterwards.  The feed-forward's output is the sum of the slabs."""
+    require_gpu()
+    _dev(h, "h", dims=2)
+    _dev(w_up, "w_up", h.dtype, 3)
+    _dev(w_down, "w_down", h.dtype, 3)
+    _dev(ids, "ids", torch.int32, 2)
+    _dev(wts, "wts", torch.float32, 2)
+    T, D = h.shape
+    E, F, _ = w_up.shape
+    K = ids.shape[1]
+    if (tuple(w_up.shape) != (E, F, D) or tuple(w_down.shape) != (E, D, F) or tuple(ids.shape) != (T, K) or tuple(wts.shape) != (T, K)
+            or not (w_up.is_contiguous() and w_down.is_contiguous() and ids.is_contiguous() and wts.is_contiguous())):
+        raise KernelError(f"moe_experts: h {tuple(h.shape)}, w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)}, ids "
+                          f"{tuple(ids.shape)} do not fit")
+    if activation not in UNARY_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
+    if (D + F) * 4 > 65536:
+        raise KernelError(f"moe_experts: width {D} and expert width {F} together are above 16,384 values")
+    y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
+    if T:
+        _check(_fn("moe", "bn_moe_experts")(_code(h.dtype), h.data_ptr(), _rows(h, "h"), w_up.data_ptr(), w_down.data_ptr(),
+                                            ids.data_ptr(), wts.data_ptr(), y.data_ptr(), T, D, F, K,
+                                            UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)), _stream()), "moe_experts")
+    return PartialSums(y)
+
+
+MOE_GROUPED_MIN_ROWS = 1 << 30      # rows from which a step's experts run as grouped products
+
+
+def moe_grouped_supported(T: int, D: int, F: int, dtype) -> bool:
+    """Whether moe_experts_grouped takes a step of T rows of these sizes and would be the faster of the two."""
+    return False
 
 
 # --------------------------------------------------------------------------------------

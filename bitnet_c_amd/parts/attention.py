@@ -12,10 +12,15 @@ stacks them, include/backend_model.h:21-22) so that one product computes them.
 A schedule entry that reads another entry's cache computes Q only.
 
 What other architectures put into the same mixer, each a parameter that is off by default; any of them takes the
-mixer to the vector kernel over pages with a row per position, in both types, and needs position "none":
+mixer to its general form: one kernel norms, rotates and stores (ops.qk_norm_store), attention reads pages with a key
+row per position and transposed values, in both types.  The general form rotates by itself (any "rope" position, in
+split-half or in neighbouring pairs, over the first rope_dims dimensions) and takes a window:
   v_head_dim     value heads of another width than the query/key heads
   qk_norm_eps    an RMSNorm over every query and every key head before they meet (tensors q_norm, k_norm [head_dim],
-                 shared by the heads, plain weights)
+                 shared by the heads, plain weights); with qk_norm_span "projection" one norm over the whole query
+                 projection and one over the whole key projection instead (q_norm [heads head_dim], k_norm
+                 [kv heads head_dim]), before the heads are split and before the rotation
+  a "rope" position with interleaved=True: pairs (2i, 2i + 1) instead of (i, i + rope_dims / 2)
   q_temp_coef, q_temp_every   the query at position p times 1 + coef * ln(floor((p + 1) / every) + 1)
   distance_bias  tensors dist_a, dist_b [heads]: dist_a[h] * ln(1 + dist_b[h] * (i - j)) is taken off the score of
                  query i and key j
@@ -42,7 +47,7 @@ class Attention(Part):
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  position: PartSpec, window: int = 0, bias: bool = False, v_head_dim: int = 0,
                  qk_norm_eps: float | None = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
-                 distance_bias: bool = False, sink: bool = False):
+                 distance_bias: bool = False, sink: bool = False, qk_norm_span: str = "head"):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
         if head_dim % 2 or head_dim < 2 or head_dim > ops.MAX_HEAD_DIM:
@@ -56,14 +61,19 @@ class Attention(Part):
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.q_temp_coef, self.q_temp_every = float(q_temp_coef), int(q_temp_every)
         self.distance_bias, self.sink = bool(distance_bias), bool(sink)
+        if qk_norm_span not in ("head", "projection"):
+            raise ValueError(f"attention: qk_norm_span {qk_norm_span!r} is neither 'head' nor 'projection'")
+        self.norm_projection = qk_norm_span == "projection"
+        if self.norm_projection and self.qk_norm_eps is None:
+            raise ValueError("attention: a norm over the whole projection needs qk_norm_eps")
         self.general = (self.vd != self.hs or self.qk_norm_eps is not None or self.q_temp_every > 0
-                        or self.distance_bias or self.sink)
+                        or self.distance_bias or self.sink or getattr(self.position, "interleaved", False))
         if self.general:
             if self.vd % 2 or self.vd < 2 or self.vd > ops.MAX_HEAD_DIM:
                 raise ValueError(f"attention: v_head_dim {self.vd} is not supported by the kernels (even, at most {ops.MAX_HEAD_DIM})")
-            if self.position.rope_dims or self.has_bias:
-                raise ValueError("attention: head norms, a query temperature, a distance bias, a sink or values of another "
-                                 "width come without a rotation and without projection biases")
+            if self.has_bias:
+                raise ValueError("attention: head norms, a query temperature, a distance bias, a sink, a rotation in neighbouring "
+                                 "pairs or values of another width come without projection biases")
             self.takes_deferred_norm = self.gives_lazy_delta = False
         self.q_norm = self.k_norm = self.dist_a = self.dist_b = None
 
@@ -79,7 +89,8 @@ class Attention(Part):
         t = {"wq": ParamSpec((self.q_dim, self.hidden)), "wk": ParamSpec((self.kv_dim, self.hidden)),
              "wv": ParamSpec((self.Hkv * self.vd, self.hidden)), "wo": ParamSpec((self.hidden, self.H * self.vd))}
         if self.qk_norm_eps is not None:
-            t.update({"q_norm": ParamSpec((self.hs,), "ones"), "k_norm": ParamSpec((self.hs,), "ones")})
+            nq, nk = (self.q_dim, self.kv_dim) if self.norm_projection else (self.hs, self.hs)
+            t.update({"q_norm": ParamSpec((nq,), "ones"), "k_norm": ParamSpec((nk,), "ones")})
         if self.distance_bias:
             t.update({"dist_a": ParamSpec((self.H,), "normal"), "dist_b": ParamSpec((self.H,), "ones")})
         if self.has_bias:
@@ -120,8 +131,9 @@ class Attention(Part):
                     and ops.can_fuse_decode(self.qkv.weight.dtype, self.H, self.Hkv, self.hs))
 
     def _forward_general(self, h, ctx, kv):
-        """Projections, head norms and temperature with the cache write (one kernel), the vector attention kernel with
-        its distance bias and sink, the output projection."""
+        """Projections; norms, rotation and temperature with the cache write (one kernel); attention with its window,
+        distance bias and sink (prompt steps on the matrix cores where the sizes allow, else the vector kernel); the
+        output projection."""
         H, Hkv, hs, vd = self.H, self.Hkv, self.hs, self.vd
         if isinstance(h, ops.DeferredNorm):
             h = h.materialize()
@@ -133,6 +145,8 @@ class Attention(Part):
             qkv[:, :self.q_dim] = self.qkv(h, rows=slice(0, self.q_dim))
         ops.qk_norm_store(qkv, ctx.positions, H, Hkv, hs, v_dim=vd, q_weight=self.q_norm, k_weight=self.k_norm,
                           eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
+                          norm_projection=self.norm_projection, inv_freq=self.position.inv_freq,
+                          rope_dims=self.position.rope_dims, rope_interleaved=getattr(self.position, "interleaved", False),
                           seq_index=ctx.seq_index if kv.writes else None, block_table=kv.block_table if kv.writes else None,
                           k_pages=kv.k_pages if kv.writes else None, v_pages=kv.v_pages if kv.writes else None,
                           v_transposed=True)

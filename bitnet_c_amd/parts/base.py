@@ -188,6 +188,15 @@ class LazyDelta:
         return self.linear(self.act)
 
 
+class NormedDelta:
+    """A part's output that goes through an RMSNorm of its own before it joins the stream (a block with output norms):
+    `delta` [T, D] in the activations' type, or ops.PartialSums (float32 slabs that are added first), and the norm.  The
+    stream adds weight * delta / rms(delta), formed in float32."""
+
+    def __init__(self, delta, norm):
+        self.delta, self.norm = delta, norm
+
+
 class ResidualStream:
     """The float32 residual stream of a step.  A part's output is held back as `pending` and
     is added by the kernel of the next norm, so the sum is formed once, in float32, without a
@@ -205,11 +214,17 @@ class ResidualStream:
         self.pending = delta
 
     def _pending_tensor(self):
+        if isinstance(self.pending, NormedDelta):
+            raise TypeError("an output with a norm of its own is added by flush() or normed()")
         if isinstance(self.pending, LazyDelta):
             self.pending = self.pending.compute()
         return self.pending
 
     def flush(self) -> torch.Tensor:
+        if isinstance(self.pending, NormedDelta):
+            from .. import ops
+            p, self.pending = self.pending, None
+            ops.add_normed_rmsnorm(self.x, p.delta, p.norm.weight, p.norm.eps)
         if self.pending is not None:
             from .. import ops
             ops.residual_add(self.x, self._pending_tensor())
@@ -222,6 +237,13 @@ class ResidualStream:
         folded around, the result is an ops.DeferredNorm instead of a tensor.  With more rows than the fused
         products take, a consumer that has a method wants_deferred_norm(ctx, rows) is asked first (ctx: the step's
         context): one that would only apply the norm the plain way gets the plain norm, in one kernel instead of two."""
+        if isinstance(self.pending, NormedDelta):
+            # the held-back output's norm, the sum and this norm in one kernel; with a choice of rows the sum comes first
+            if rows is None and getattr(norm, "normed_delta", False):
+                from .. import ops
+                p, self.pending = self.pending, None
+                return ops.add_normed_rmsnorm(self.x, p.delta, p.norm.weight, p.norm.eps, norm.weight, norm.eps, out_dtype)
+            self.flush()
         if (rows is None and isinstance(self.pending, LazyDelta) and getattr(consumer, "takes_deferred_norm", False)
                 and getattr(norm, "deferrable", False)):
             deferred = self.pending.linear.into_stream(self.pending.act, self.x, norm.weight, norm.eps)

@@ -17,6 +17,7 @@ class RMSNorm(Part):
     prompt_capturable = True    # a prompt step is read from the context's device tensors alone
     deferrable = True        # a product may fold this norm around itself (weight and eps are all it needs)
     takes_partial_sums = True    # apply() accepts ops.PartialSums as the delta
+    normed_delta = True          # weight and eps are all that ops.add_normed_rmsnorm needs: it may be a block's output norm
 
     def __init__(self, dim: int, eps: float, scalar: bool = False):
         self.dim, self.eps, self.scalar = int(dim), float(eps), bool(scalar)

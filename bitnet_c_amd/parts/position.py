@@ -52,9 +52,11 @@ class PositionEncoding(Part):
         cache write itself: a rotation of the whole head with these frequencies, or none."""
         if self.rope_dims == 0:
             return True, None
-        return self.rope_dims == hs, self.inv_freq
+        return self.rope_dims == hs and not getattr(self, "interleaved", False), self.inv_freq
 
     def encode_and_store(self, qkv, ctx, H, Hkv, hs, kv) -> None:
+        if getattr(self, "interleaved", False):
+            raise ValueError("a rotation in neighbouring pairs is done by the attention mixer's general form")
         ops.rope_kv_write(qkv, ctx.positions, H, Hkv, hs, inv_freq=self.inv_freq, rope_dims=self.rope_dims,
                           seq_index=ctx.seq_index if kv.writes else None,
                           block_table=kv.block_table if kv.writes else None,
@@ -67,8 +69,11 @@ class PositionEncoding(Part):
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
     prompt_capturable = True    # a prompt step is read from the context's device tensors alone
-    def __init__(self, head_dim: int, theta: float, rope_dims: int = 0, scaling=None):
+    def __init__(self, head_dim: int, theta: float, rope_dims: int = 0, scaling=None, interleaved: bool = False):
+        """interleaved: the rotated pairs are neighbours, (2i, 2i + 1), instead of (i, i + rope_dims / 2).  Only the
+        attention mixer's general form rotates that way (it does the rotation itself, ops.qk_norm_store)."""
         self.head_dim = int(head_dim)
+        self.interleaved = bool(interleaved)
         self.rope_dims = int(rope_dims) or self.head_dim
         if self.rope_dims % 2 or self.rope_dims > self.head_dim:
             raise ValueError(f"rope: rope_dims {self.rope_dims} must be even and at most head_dim {head_dim}")

@@ -4,7 +4,9 @@
 // ([page, kv head, BN_PAGE, hs]), values transposed ([page, kv head, vd, BN_PAGE]): both operands of both products are
 // then 16 consecutive bytes a lane, straight from the pages (no shared memory, no barrier: a wave is on its own).
 //
-// A wave owns one tile of up to 16 query tokens of one head and walks the keys 0 .. last query in blocks of 32:
+// A wave owns one tile of up to 16 query tokens of one head and walks the keys 0 .. last query in blocks of 32 (with a
+// window w > 0 a query at position i sees the keys i - w + 1 .. i only, and the walk begins at the block of the tile's
+// first visible key):
 //   S^T = K . Q^T      two tiles of 16 keys x 16 queries; tile h holds the block's keys 8 (i / 4) + 4 h + i % 4 in its
 //                      row i, so that lane group g ends up with the scores of keys 8 g .. 8 g + 7 of its query column:
 //                      what the second product wants from it as its operand, without any exchange
@@ -35,6 +37,7 @@ struct GenArgs {
     int q_stride, out_stride, bt_stride, H, Hkv;
     float scale;
     int sink;
+    int window;               // 0: every earlier key; else the last `window` positions, the query's own included
 };
 
 __device__ __forceinline__ bf16x8 ag_ld16(const bf16* p) {
@@ -80,9 +83,11 @@ __global__ __launch_bounds__(AG_WAVES * BN_WAVE) void attn_general_prompt_kernel
 #pragma unroll
         for (int c = 0; c < DC; ++c) { kn0[c] = ag_ld16(kbase + 32 * c); kn1[c] = ag_ld16(kbase + 4 * HS + 32 * c); }
     };
-    ask_keys(0);
+    const int k_lo = a.window > 0 ? max(0, pos0 - a.window + 1) & ~31 : 0;      // the block of the first key any row sees
+    const int q_lo = a.window > 0 ? qpos - a.window : -1;                        // keys at or below this are out of sight
+    ask_keys(k_lo);
     const int last_block = ((k_hi - 1) / 32) * 32;
-    for (int kb = 0; kb < k_hi; kb += 32) {
+    for (int kb = k_lo; kb < k_hi; kb += 32) {
         const int page = a.block_table[(size_t)seq * a.bt_stride + kb / BN_PAGE];
         const int off = kb % BN_PAGE;
         const bf16* vbase = a.v_pages + (((size_t)page * a.Hkv + kvh) * VD + i) * BN_PAGE + off + 8 * g;
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(AG_WAVES * BN_WAVE) void attn_general_prompt_kernel
             const int key = kb + 8 * g + e;
             float v = (e < 4 ? st0[e & 3] : st1[e & 3]) * scale2;
             if (a.dist_a) v -= ba * __log2f(1.0f + bb * (float)(qpos - key));     // a ln(x) log2(e) = a log2(x)
-            if (!col_ok || key > qpos || key >= k_hi) v = -INFINITY;
+            if (!col_ok || key > qpos || key >= k_hi || key <= q_lo) v = -INFINITY;
             s[e] = v;
             mx = fmaxf(mx, v);
         }
@@ -196,8 +201,8 @@ static int ag_launch_dt(const GenArgs& a, int vd, dim3 grid, hipStream_t s) {
 extern "C" int bn_attn_general_prompt(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                                       const void* v_pages, const int* block_table, int bt_stride, const int* tiles, int n_tiles,
                                       int H, int Hkv, int hs, int vd, float scale, const float* dist_a, const float* dist_b,
-                                      int sink, hipStream_t s) {
-    if (n_tiles <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || !bn_attn_general_supports(hs, vd)) return BN_ERR_ARG;
+                                      int sink, int window, hipStream_t s) {
+    if (n_tiles <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || window < 0 || !bn_attn_general_supports(hs, vd)) return BN_ERR_ARG;
     if (!q || !out || !k_pages || !v_pages || !block_table || !tiles || (dist_a == nullptr) != (dist_b == nullptr)) return BN_ERR_ARG;
     if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) || ((uintptr_t)out & 7))
         return BN_ERR_ARG;
@@ -205,7 +210,7 @@ extern "C" int bn_attn_general_prompt(const void* q, int q_stride, void* out, in
     a.q = (const bf16*)q; a.out = (bf16*)out; a.k_pages = (const bf16*)k_pages; a.v_pages = (const bf16*)v_pages;
     a.block_table = block_table; a.tiles = tiles; a.dist_a = dist_a; a.dist_b = dist_b;
     a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv;
-    a.scale = scale; a.sink = sink ? 1 : 0;
+    a.scale = scale; a.sink = sink ? 1 : 0; a.window = window;
     const dim3 grid(n_tiles, (H + AG_WAVES - 1) / AG_WAVES);
     switch (hs / 32) {
         case 1: return ag_launch_dt<1>(a, vd, grid, s);

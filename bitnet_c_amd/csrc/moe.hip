@@ -68,6 +68,7 @@ __global__ __launch_bounds__(BN_WAVE) void moe_route_kernel(RouteArgs a) {
             const int oa = __shfl_xor(at, o, BN_WAVE);
             if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
         }
+        if (at >= a.E) at = k;                           // a row of NaNs (a padding row's garbage): still an expert that exists
 #pragma unroll
         for (int j = 0; j < MOE_PER_LANE; ++j)
             if (at == lane + BN_WAVE * j) z[j] = -INFINITY;
@@ -162,5 +163,174 @@ extern "C" int bn_moe_experts(int dtype, const void* h, int ld, const void* w_up
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_pair_kernel<float>, grid, block, shm, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_pair_kernel<bf16>, grid, block, shm, s, a);
     else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- grouped products on the matrix cores (bf16) ---------------------------------------------------------------------
+// The pairs of a step are ordered by expert and cut into tiles of up to MOE_TILE rows of one expert; a workgroup takes one
+// tile and 64 columns of the product, its four waves 16 columns each: a wave loads a 16 x 32 piece of the expert's matrix
+// once and uses it for both 16-row halves of the tile (v_mfma_f32_16x16x32_bf16; the matrix as the first operand, so that
+// a lane ends up with four consecutive result columns of one row: one store).  Operands come straight from memory, 16 bytes
+// a lane; everything that a tile needs to know lies in device memory, so the launches do not depend on the routing.
+#define MOE_TILE 32
+#define MOE_PLAN_THREADS 1024
+
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
+typedef __attribute__((ext_vector_type(8))) float moe_f32x8;
+typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
+
+// order [T K]: the pairs (t K + j) by expert; tiles [max_tiles][3] = expert, first place in `order`, rows; n_tiles [1]
+__global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* __restrict__ ids, int n_pairs, int E,
+                                                                    int* __restrict__ order, int* __restrict__ tiles,
+                                                                    int* __restrict__ n_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS + 1], tile0[MOE_MAX_EXPERTS + 1];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, tl = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = at; tile0[e] = tl;
+            at += count[e];
+            tl += (count[e] + MOE_TILE - 1) / MOE_TILE;
+        }
+        first[E] = at; tile0[E] = tl;
+        n_tiles[0] = tl;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        const int n = count[e];
+        for (int r = 0, k = tile0[e]; r < n; r += MOE_TILE, ++k) {
+            tiles[3 * k] = e; tiles[3 * k + 1] = first[e] + r; tiles[3 * k + 2] = min(MOE_TILE, n - r);
+        }
+        count[e] = 0;                                    // now the cursor of the scatter
+    }
+    __syncthreads();
+    // the places inside an expert's run are handed out in whatever order the lanes arrive: a row's result does not depend
+    // on its place
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = ids[p];
+        order[first[e] + atomicAdd(&count[e], 1)] = p;
+    }
+}
+
+struct GroupedArgs {
+    const bf16* x;            // up: h [T, ldx]; down: hidden [pairs, F] in the order of `order`
+    const bf16* w;            // up: [E, F, D]; down: [E, D, F]
+    bf16* hidden;             // up's result
+    float* y;                 // down's result [K, T, D]
+    const int* order;
+    const int* tiles;
+    const int* n_tiles;
+    const float* wts;         // [T, K]
+    int ldx, T, D, F, K, act, weight_on_input;
+};
+
+__device__ __forceinline__ moe_bf16x8 moe_ld16(const bf16* p) {
+    return __builtin_bit_cast(moe_bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+// hidden[place] = act(W_up[e] (w h[t]))  for the rows of a tile; N = F columns, the sum runs over D
+__global__ __launch_bounds__(256) void moe_grouped_up_kernel(GroupedArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= a.n_tiles[0]) return;
+    const int e = a.tiles[3 * tile], start = a.tiles[3 * tile + 1], rows = a.tiles[3 * tile + 2];
+    const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+    const int f0 = blockIdx.y * 64 + 16 * (threadIdx.x >> 6);
+    if (f0 >= a.F) return;
+    const bf16* wrow = a.w + ((size_t)e * a.F + f0 + i) * a.D + 8 * g;
+    const bf16* xrow[2];
+    float sc[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const int pair = a.order[start + min(16 * s + i, rows - 1)];
+        xrow[s] = a.x + (size_t)(pair / a.K) * a.ldx + 8 * g;
+        sc[s] = a.weight_on_input ? a.wts[pair] : 1.0f;
+    }
+    moe_f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int c = 0; c < a.D; c += 32) {
+        const moe_bf16x8 wf = moe_ld16(wrow + c);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (s == 1 && rows <= 16) break;
+            moe_bf16x8 xf = moe_ld16(xrow[s] + c);
+            if (a.weight_on_input) {                     // the expert reads w h, rounded to the activations' type
+                moe_f32x8 xv = __builtin_convertvector(xf, moe_f32x8);
+                xv *= sc[s];
+                xf = __builtin_convertvector(xv, moe_bf16x8);
+            }
+            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[s], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const int r = 16 * s + i;
+        if (r >= rows) continue;
+        bf16 o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = __float2bfloat16(bn_unary_act(acc[s][k], a.act));
+        uint2 pk;
+        pk.x = (uint32_t)__builtin_bit_cast(unsigned short, o[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, o[1]) << 16);
+        pk.y = (uint32_t)__builtin_bit_cast(unsigned short, o[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, o[3]) << 16);
+        *reinterpret_cast<uint2*>(a.hidden + (size_t)(start + r) * a.F + f0 + 4 * g) = pk;
+    }
+}
+
+// y[j][t] = W_down[e] hidden[place] (times w when the weight multiplies the output); N = D columns, the sum runs over F
+__global__ __launch_bounds__(256) void moe_grouped_down_kernel(GroupedArgs a) {
+    const int tile = blockIdx.x;
+    if (tile >= a.n_tiles[0]) return;
+    const int e = a.tiles[3 * tile], start = a.tiles[3 * tile + 1], rows = a.tiles[3 * tile + 2];
+    const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+    const int d0 = blockIdx.y * 64 + 16 * (threadIdx.x >> 6);
+    if (d0 >= a.D) return;
+    const bf16* wrow = a.w + ((size_t)e * a.D + d0 + i) * a.F + 8 * g;
+    const bf16* xrow[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) xrow[s] = a.x + (size_t)(start + min(16 * s + i, rows - 1)) * a.F + 8 * g;
+    moe_f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int c = 0; c < a.F; c += 32) {
+        const moe_bf16x8 wf = moe_ld16(wrow + c);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (s == 1 && rows <= 16) break;
+            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, moe_ld16(xrow[s] + c), acc[s], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const int r = 16 * s + i;
+        if (r >= rows) continue;
+        const int pair = a.order[start + r], t = pair / a.K, j = pair - t * a.K;
+        const float f = a.weight_on_input ? 1.0f : a.wts[pair];
+        float4 o = make_float4(acc[s][0] * f, acc[s][1] * f, acc[s][2] * f, acc[s][3] * f);
+        *reinterpret_cast<float4*>(a.y + ((size_t)j * a.T + t) * a.D + d0 + 4 * g) = o;
+    }
+}
+
+// 1 if the grouped products take these sizes (the sums run over whole chunks of 32, the columns come in sixteens)
+extern "C" int bn_moe_grouped_supports(int D, int F) { return (D > 0 && F > 0 && D % 32 == 0 && F % 32 == 0) ? 1 : 0; }
+extern "C" int bn_moe_grouped_tiles(int n_pairs, int E) { return (n_pairs + MOE_TILE - 1) / MOE_TILE + E; }
+
+// work: int32 [n_pairs + 3 max_tiles + 1] (order, tiles, n_tiles); hidden: bf16 [n_pairs, F]
+extern "C" int bn_moe_grouped(const void* h, int ld, const void* w_up, const void* w_down, const int* ids, const float* wts,
+                              float* y, int* work, void* hidden, int n_tokens, int D, int F, int E, int K, int act,
+                              int weight_on_input, hipStream_t s) {
+    if (n_tokens <= 0 || K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || !bn_moe_grouped_supports(D, F) || ld < D || ld % 8) return BN_ERR_ARG;
+    if (act < 0 || act >= BN_UNARY_KINDS || !h || !w_up || !w_down || !ids || !wts || !y || !work || !hidden) return BN_ERR_ARG;
+    if ((((uintptr_t)h | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)y | (uintptr_t)hidden) & 15)) return BN_ERR_ARG;
+    const int n_pairs = n_tokens * K, max_tiles = bn_moe_grouped_tiles(n_pairs, E);
+    int* order = work;
+    int* tiles = work + n_pairs;
+    int* n_tiles = tiles + 3 * max_tiles;
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(MOE_PLAN_THREADS), 0, s, ids, n_pairs, E, order, tiles, n_tiles);
+    GroupedArgs a;
+    a.x = (const bf16*)h; a.w = (const bf16*)w_up; a.hidden = (bf16*)hidden; a.y = y; a.order = order; a.tiles = tiles;
+    a.n_tiles = n_tiles; a.wts = wts; a.ldx = ld; a.T = n_tokens; a.D = D; a.F = F; a.K = K; a.act = act;
+    a.weight_on_input = weight_on_input ? 1 : 0;
+    hipLaunchKernelGGL(moe_grouped_up_kernel, dim3(max_tiles, (F + 63) / 64), dim3(256), 0, s, a);
+    a.x = (const bf16*)hidden; a.w = (const bf16*)w_down;
+    hipLaunchKernelGGL(moe_grouped_down_kernel, dim3(max_tiles, (D + 63) / 64), dim3(256), 0, s, a);
     return bn_launch_status();
 }

@@ -69,11 +69,15 @@ _SIGNATURES = {
                          c_void_p],
         "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                            c_int, c_int, c_void_p],
+        "bn_moe_grouped_supports": [c_int, c_int],
+        "bn_moe_grouped_tiles": [c_int, c_int],
+        "bn_moe_grouped": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                           c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attn_mfma_general": {
         "bn_attn_general_supports": [c_int, c_int],
         "bn_attn_general_prompt": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p],
+                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
     },
     "state_mixers": {
         "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
@@ -1391,9 +1395,10 @@ def attention_general_supported(dtype, hs: int, v_dim: int) -> bool:
 
 def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                              block_table: torch.Tensor, H: int, Hkv: int, hs: int, v_dim: int, scale: float, tiles: torch.Tensor,
-                             *, distance_bias=None, sink: bool = False) -> None:
+                             *, distance_bias=None, sink: bool = False, window: int = 0) -> None:
     """Causal prompt attention on the matrix cores for what attention() leaves to the vector kernel: bf16, keys 32, 64,
-    96, 128 or 256 wide, values of a width of their own from the same list, a distance bias and a sink (as attention()'s).
+    96, 128 or 256 wide, values of a width of their own from the same list, a distance bias and a sink (as attention()'s),
+    a window (> 0: a query sees the last `window` positions, its own included).  qkv's row stride is a multiple of 8.
     Pages: keys a row per position, values transposed.  tiles [n, 4] int32: (sequence, first row, rows <= 16, position of
     the first), any order, tiles of no rows skipped.  out [T, H v_dim]."""
     require_gpu()
@@ -1416,13 +1421,15 @@ def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torc
             _dev(t, nm, torch.float32, 1)
             if t.numel() != H or not t.is_contiguous():
                 raise KernelError(f"attention_general_prompt: {nm} must hold one float32 per head")
+    if window < 0 or _rows(qkv, "qkv") % 8 or qkv.data_ptr() % 16:
+        raise KernelError(f"attention_general_prompt: window {window} / row stride {_rows(qkv, 'qkv')} (a multiple of 8, 16-byte aligned)")
     if T == 0 or tiles.shape[0] == 0:
         return
     _check(_fn("attn_mfma_general", "bn_attn_general_prompt")(
         qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * v_dim, k_pages.data_ptr(), v_pages.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], tiles.data_ptr(), tiles.shape[0], H, Hkv, hs, v_dim, float(scale),
-        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), _stream()),
-        "attention_general_prompt")
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), int(window),
+        _stream()), "attention_general_prompt")
 
 
 # --------------------------------------------------------------------------------------
@@ -1824,12 +1831,52 @@ def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: 
     return PartialSums(y)
 
 
-MOE_GROUPED_MIN_ROWS = 1 << 30      # rows from which a step's experts run as grouped products
+MOE_GROUPED_MIN_ROWS = 17           # rows from which a bf16 step's experts run as grouped products (below: a pair a workgroup)
+MOE_TILE = _build.header_constant("MOE_TILE", "moe.hip")
 
 
 def moe_grouped_supported(T: int, D: int, F: int, dtype) -> bool:
-    """Whether moe_experts_grouped takes a step of T rows of these sizes and would be the faster of the two."""
-    return False
+    """Whether moe_experts_grouped takes a step of T rows of these sizes and is the faster of the two: bf16, sums over whole
+    chunks of 32 (bn_moe_grouped_supports, answered here so that asking loads no kernel), and enough rows for experts to
+    be shared."""
+    return dtype == torch.bfloat16 and T >= MOE_GROUPED_MIN_ROWS and D % 32 == 0 and F % 32 == 0
+
+
+def moe_experts_grouped(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
+                        activation: str = "relu2", weight_on_input: bool = True) -> PartialSums:
+    """What moe_experts computes, for bf16 steps of many rows: the (token, choice) pairs are ordered by expert on the
+    device and cut into tiles of up to MOE_TILE rows of one expert, and both products run on the matrix cores over those
+    tiles.  Nothing comes back to the host; the launches' sizes depend on the step's shape alone."""
+    require_gpu()
+    _dev(h, "h", torch.bfloat16, 2)
+    _dev(w_up, "w_up", torch.bfloat16, 3)
+    _dev(w_down, "w_down", torch.bfloat16, 3)
+    _dev(ids, "ids", torch.int32, 2)
+    _dev(wts, "wts", torch.float32, 2)
+    T, D = h.shape
+    E, F, _ = w_up.shape
+    K = ids.shape[1]
+    if (tuple(w_up.shape) != (E, F, D) or tuple(w_down.shape) != (E, D, F) or tuple(ids.shape) != (T, K) or tuple(wts.shape) != (T, K)
+            or not (w_up.is_contiguous() and w_down.is_contiguous() and ids.is_contiguous() and wts.is_contiguous())):
+        raise KernelError(f"moe_experts_grouped: h {tuple(h.shape)}, w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)}, ids "
+                          f"{tuple(ids.shape)} do not fit")
+    if activation not in UNARY_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
+    ld = _rows(h, "h")
+    if D % 32 or F % 32 or E > MOE_MAX_EXPERTS or ld % 8 or h.data_ptr() % 16:
+        raise KernelError(f"moe_experts_grouped: widths {D} and {F} must be multiples of 32, rows 16-byte aligned, at most "
+                          f"{MOE_MAX_EXPERTS} experts")
+    y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
+    if T == 0:
+        return PartialSums(y)
+    max_tiles = -(-T * K // MOE_TILE) + E
+    work = torch.empty((T * K + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+    hidden = torch.empty((T * K, F), dtype=torch.bfloat16, device=h.device)
+    _check(_fn("moe", "bn_moe_grouped")(h.data_ptr(), ld, w_up.data_ptr(), w_down.data_ptr(), ids.data_ptr(), wts.data_ptr(),
+                                        y.data_ptr(), work.data_ptr(), hidden.data_ptr(), T, D, F, E, K,
+                                        UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)), _stream()),
+           "moe_experts_grouped")
+    return PartialSums(y)
 
 
 # --------------------------------------------------------------------------------------

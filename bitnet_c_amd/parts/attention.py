@@ -159,9 +159,11 @@ class Attention(Part):
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=True, blocked=False,
                           v_dim=vd, distance_bias=bias, sink=self.sink)
-        elif not self.window and ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES:
+        elif (ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES and width % 8 == 0
+              and qkv.data_ptr() % 16 == 0):
             ops.attention_general_prompt(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, vd, self.scale,
-                                         ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self.sink)
+                                         ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self.sink,
+                                         window=self.window)
         else:
             _, _, qt = ops.attention_row_shape(H, Hkv, False)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,

@@ -169,18 +169,57 @@ KERNEL_WORKLOADS = {"skinny": _kernel_skinny, "gemm": _kernel_gemm, "attention_p
 
 
 # ---- another design beside the Llama-style decoder at equal size (--design) ----------------------------------------
-# Layer sizes that resemble real models: width, feed-forward, 64-wide recurrence heads, attention heads of 128.
+# Layer sizes that resemble real models: width, feed-forward, 64-wide recurrence heads, attention heads of 128; for the
+# designs with windows, latent attention and experts: the window, the rotated part of a head, the latent's width, and
+# experts whose active weights per token equal the gated feed-forward's (top * 2 * expert_ff = 3 * gated ff).
 DESIGN_SIZES = {
     "2048": dict(width=2048, ff=8192, rec_heads=32, rec_dim=64, rank=64, heads=16, kv_heads=4, dim=128, right=2048,
-                 vocab=32000, layers=12),
+                 vocab=32000, layers=12, window=1024, rot_dims=64, kv_rank=256, experts=16, top=2),
     "4096": dict(width=4096, ff=16384, rec_heads=64, rec_dim=64, rank=128, heads=32, kv_heads=8, dim=128, right=4096,
-                 vocab=32000, layers=9),
+                 vocab=32000, layers=9, window=1024, rot_dims=64, kv_rank=256, experts=16, top=2),
 }
 
 
-def _design_configs(z):
-    """(Sunusun config.json, Llama config.json) of equal width, layers, attention heads and (nearly) equal weight bytes:
-    two recurrent layers, then one parallel layer, repeated; the gated feed-forward is 2/3 as wide as the dense one."""
+def _llama_config(z):
+    return dict(model_type="llama", vocab_size=z["vocab"], hidden_size=z["width"],
+                intermediate_size=(2 * z["ff"] // 3 + 255) // 256 * 256, num_hidden_layers=z["layers"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
+
+
+def _sonodra_configs(z):
+    """(Sonodra config.json, Llama config.json) of equal width, layers and attention heads, and equal weight bytes read per
+    token: two windowed attention layers, then a latent attention layer (every second one reading the latent vectors of the
+    one before it), repeated; the first layer's feed-forward is the gated one of the Llama-style decoder, the others choose
+    `top` of `experts` experts whose two matrices together are as large as the gated unit's three."""
+    gated = _llama_config(z)["intermediate_size"]
+    moe = dict(kind="moe", expert=dict(ff=3 * gated // (2 * z["top"]) // 32 * 32), router=dict(experts=z["experts"], top=z["top"]))
+    att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+               mask=dict(size=z["window"]), rot=dict(base=10000.0, dims=z["rot_dims"]))
+    lat = dict(heads=z["heads"], dim=z["dim"], vdim=z["dim"], kv_rank=z["kv_rank"], scale=z["dim"] ** -0.5)
+    layers, first_latent = [], None
+    for i in range(z["layers"]):
+        mlp = dict(kind="dense", ff=gated) if i == 0 else moe
+        if i % 3 != 2:
+            layers.append(dict(type="attention", mixer=att, mlp=mlp))
+        elif first_latent is None or len([L for L in layers if L["type"] == "latent_attention"]) % 2 == 0:
+            first_latent = i
+            layers.append(dict(type="latent_attention", mixer=lat, mlp=mlp))
+        else:
+            layers.append(dict(type="latent_attention", mixer=dict(lat, kv_from=first_latent), mlp=mlp))
+    son = dict(architecture="Sonodra", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6), layers=layers)
+    return son, _llama_config(z)
+
+
+def _design_configs(design, z):
+    """(the design's config.json, Llama config.json) of equal width, layers, attention heads and (nearly) equal weight bytes."""
+    if design == "sonodra":
+        return _sonodra_configs(z)
+    return _sunusun_configs(z)
+
+
+def _sunusun_configs(z):
+    """Two recurrent layers, then one parallel layer, repeated; the gated feed-forward is 2/3 as wide as the dense one."""
     wkv = dict(type="wkv", mixer=dict(heads=z["rec_heads"], dim=z["rec_dim"], decay_rank=z["rank"]),
                mlp=dict(kind="dense", ff=z["ff"]))
     par = dict(type="parallel", mlp=dict(kind="dense", ff=z["ff"]), mixer=dict(
@@ -188,11 +227,7 @@ def _design_configs(z):
                   q_temp=dict(coef=0.1, every=256)), right=dict(width=z["right"])))
     sun = dict(architecture="Sunusun", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6), logit_scale=1.0,
                layers=[par if i % 3 == 2 else wkv for i in range(z["layers"])])
-    llama = dict(model_type="llama", vocab_size=z["vocab"], hidden_size=z["width"],
-                 intermediate_size=(2 * z["ff"] // 3 + 255) // 256 * 256, num_hidden_layers=z["layers"],
-                 num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
-                 max_position_embeddings=8192, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False)
-    return sun, llama
+    return sun, _llama_config(z)
 
 
 def bench_design(args) -> int:
@@ -211,7 +246,7 @@ def bench_design(args) -> int:
     PREFILL, lens = args.prefill_tokens, (256, 1024)
     out = {"design": args.design, "size": args.design_size, "sizes": z, "dtype": "bf16", "steps": args.steps, "warmup": args.warmup,
            "prefill_tokens": PREFILL, "decode_prompt_lens": list(lens), "data": "synthetic: random N(0,0.02) weights, uniform token ids"}
-    for name, raw in zip((args.design, "llama"), _design_configs(z)):
+    for name, raw in zip((args.design, "llama"), _design_configs(args.design, z)):
         arch = architecture_for(raw)
         cfg = arch.config_cls.from_dict(raw)
         plan = arch.build_plan(cfg)
@@ -286,7 +321,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=0, help="longest sequence (default: the shape's)")
     ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the measured prompt step")
-    ap.add_argument("--design", choices=["sunusun"], default=None,
+    ap.add_argument("--design", choices=["sunusun", "sonodra"], default=None,
                     help="instead of the benchmark: prefill and decode of this design beside the Llama-style decoder of equal "
                          "width, heads, layers and weight bytes, at the sizes of --design-size (random weights; one JSON line)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="2048")

@@ -3,9 +3,10 @@
 //   bn_moe_route     router logits z = W_r h in float32 (one wave a token), scores sigmoid(z) or softmax(z), the top_k
 //                    largest (ties: the lower index), optionally divided by their sum -> expert ids and weights [T, top_k]
 //   bn_moe_experts   for every (token, choice) pair: y = W_down[e] act(W_up[e] (w h)) when the weight multiplies the
-//                    expert's input, w * W_down[e] act(W_up[e] h) when it multiplies the output; one workgroup a pair, which
-//                    reads the expert's two matrices once.  The products accumulate in float32; the scaled input and the
-//                    hidden vector are rounded to the activations' type as a product of that type would see them.
+//                    expert's input, w * W_down[e] act(W_up[e] h) when it multiplies the output; a pair reads its expert's
+//                    two matrices once, their rows spread over workgroups.  The products accumulate in float32; the scaled
+//                    input and the hidden vector are rounded to the activations' type as a product of that type would
+//                    see them.
 //   bn_moe_plan      pairs ordered by expert, and tiles of up to MOE_TILE rows of one expert each, for the grouped products
 //   bn_moe_grouped   (bf16) the same two products on the matrix cores over those tiles: a tile's rows share an expert
 // The outputs of a token's choices land in slab j of y [top_k, T, D] (float32) and are added by whoever consumes y.
@@ -104,8 +105,13 @@ extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, i
     return bn_launch_status();
 }
 
-// ---- one workgroup a (token, choice) pair -----------------------------------------------------------------------------
+// ---- a (token, choice) pair at a time ----------------------------------------------------------------------------------
+// Steps of few rows: every pair reads its expert's two matrices once, and the rows of a matrix are spread over many
+// workgroups so that one pair alone fills the chip (two launches: the hidden vector, then the output).  A workgroup stages
+// the pair's input vector in shared memory as float32, each of its waves takes MOE_PAIR_ROWS / 4 rows of the matrix, a row
+// as 16-byte loads across the lanes (bf16 rows of whole 8-element groups) or element by element, and sums in float32.
 #define MOE_PAIR_THREADS 256
+#define MOE_PAIR_ROWS 16
 
 struct PairArgs {
     const void* h;            // [T, ld]
@@ -113,56 +119,94 @@ struct PairArgs {
     const void* w_down;       // [E, D, F]
     const int* ids;           // [T, K]
     const float* wts;         // [T, K]
+    float* hidden;            // [T K, F] float32 holding values of the activations' type
     float* y;                 // [K, T, D]
-    int ld, T, D, F, K, act, weight_on_input;
+    int ld, T, D, F, K, act, weight_on_input;      // T: the rows of a slab of y
 };
 
+// sum over n of x[i] w[i]: x in shared memory, w a row in global memory; every lane gets the sum
 template <typename T>
-__global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_kernel(PairArgs a) {
-    extern __shared__ float sh[];                        // x [D], then hidden [F]
-    float* xs = sh;
-    float* hid = sh + a.D;
-    const int pair = blockIdx.x, t = pair / a.K, j = pair - t * a.K;
-    const int lane = threadIdx.x & (BN_WAVE - 1), wave = threadIdx.x / BN_WAVE, n_waves = MOE_PAIR_THREADS / BN_WAVE;
+__device__ __forceinline__ float moe_row_dot(const T* __restrict__ w, const float* __restrict__ x, int n, int lane) {
+    float s = 0.f;
+    for (int i = lane; i < n; i += BN_WAVE) s = fmaf(x[i], to_f32(w[i]), s);
+    return wave_sum(s);
+}
+template <>
+__device__ __forceinline__ float moe_row_dot<bf16>(const bf16* __restrict__ w, const float* __restrict__ x, int n, int lane) {
+    float s = 0.f;
+    if (n % 8 == 0 && ((uintptr_t)w & 15) == 0) {
+        for (int i = 8 * lane; i < n; i += 8 * BN_WAVE) {
+            const uint4 p = *reinterpret_cast<const uint4*>(w + i);
+            const float4 a = *reinterpret_cast<const float4*>(x + i), b = *reinterpret_cast<const float4*>(x + i + 4);
+            s = fmaf(a.x, bf16lo_to_f32(p.x), s); s = fmaf(a.y, bf16hi_to_f32(p.x), s);
+            s = fmaf(a.z, bf16lo_to_f32(p.y), s); s = fmaf(a.w, bf16hi_to_f32(p.y), s);
+            s = fmaf(b.x, bf16lo_to_f32(p.z), s); s = fmaf(b.y, bf16hi_to_f32(p.z), s);
+            s = fmaf(b.z, bf16lo_to_f32(p.w), s); s = fmaf(b.w, bf16hi_to_f32(p.w), s);
+        }
+    } else {
+        for (int i = lane; i < n; i += BN_WAVE) s = fmaf(x[i], to_f32(w[i]), s);
+    }
+    return wave_sum(s);
+}
+
+// hidden[pair][f] = act(W_up[e][f] . (w h[t])) for the workgroup's rows f
+template <typename T>
+__global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_up_kernel(PairArgs a) {
+    extern __shared__ __align__(16) float xs[];          // [D]
+    const int pair = blockIdx.y, t = pair / a.K;
+    const int lane = threadIdx.x & (BN_WAVE - 1), wave = threadIdx.x / BN_WAVE;
     const int e = a.ids[pair];
-    const float wt = a.wts[pair];
-    const float in_scale = a.weight_on_input ? wt : 1.0f, out_scale = a.weight_on_input ? 1.0f : wt;
+    const float in_scale = a.weight_on_input ? a.wts[pair] : 1.0f;
     const T* h = reinterpret_cast<const T*>(a.h) + (size_t)t * a.ld;
     for (int d = threadIdx.x; d < a.D; d += MOE_PAIR_THREADS) xs[d] = to_f32(from_f32<T>(to_f32(h[d]) * in_scale));
     __syncthreads();
     const T* wu = reinterpret_cast<const T*>(a.w_up) + (size_t)e * a.F * a.D;
-    for (int f = wave; f < a.F; f += n_waves) {
-        const T* w = wu + (size_t)f * a.D;
-        float s = 0.f;
-        for (int d = lane; d < a.D; d += BN_WAVE) s = fmaf(xs[d], to_f32(w[d]), s);
-        s = wave_sum(s);
-        if (lane == 0) hid[f] = to_f32(from_f32<T>(bn_unary_act(s, a.act)));
+    const int f0 = blockIdx.x * MOE_PAIR_ROWS;
+    for (int f = f0 + wave; f < min(f0 + MOE_PAIR_ROWS, a.F); f += MOE_PAIR_THREADS / BN_WAVE) {
+        const float s = moe_row_dot<T>(wu + (size_t)f * a.D, xs, a.D, lane);
+        if (lane == 0) a.hidden[(size_t)pair * a.F + f] = to_f32(from_f32<T>(bn_unary_act(s, a.act)));
     }
+}
+
+// y[j][t][d] = W_down[e][d] . hidden[pair] (times w when the weight multiplies the output) for the workgroup's rows d
+template <typename T>
+__global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_down_kernel(PairArgs a) {
+    extern __shared__ __align__(16) float hid[];         // [F]
+    const int pair = blockIdx.y, t = pair / a.K, j = pair - t * a.K;
+    const int lane = threadIdx.x & (BN_WAVE - 1), wave = threadIdx.x / BN_WAVE;
+    const int e = a.ids[pair];
+    const float out_scale = a.weight_on_input ? 1.0f : a.wts[pair];
+    for (int f = threadIdx.x; f < a.F; f += MOE_PAIR_THREADS) hid[f] = a.hidden[(size_t)pair * a.F + f];
     __syncthreads();
     const T* wd = reinterpret_cast<const T*>(a.w_down) + (size_t)e * a.D * a.F;
     float* y = a.y + ((size_t)j * a.T + t) * a.D;
-    for (int d = wave; d < a.D; d += n_waves) {
-        const T* w = wd + (size_t)d * a.F;
-        float s = 0.f;
-        for (int f = lane; f < a.F; f += BN_WAVE) s = fmaf(hid[f], to_f32(w[f]), s);
-        s = wave_sum(s);
+    const int d0 = blockIdx.x * MOE_PAIR_ROWS;
+    for (int d = d0 + wave; d < min(d0 + MOE_PAIR_ROWS, a.D); d += MOE_PAIR_THREADS / BN_WAVE) {
+        const float s = moe_row_dot<T>(wd + (size_t)d * a.F, hid, a.F, lane);
         if (lane == 0) y[d] = s * out_scale;
     }
 }
 
+// hidden: float32 work space [n_tokens K, F]; y_rows: the rows of a slab of y (>= n_tokens: the call may take a run of a
+// step's tokens, y then points at the run's first row of slab 0)
 extern "C" int bn_moe_experts(int dtype, const void* h, int ld, const void* w_up, const void* w_down, const int* ids,
-                              const float* wts, float* y, int n_tokens, int D, int F, int K, int act, int weight_on_input,
-                              hipStream_t s) {
-    if (n_tokens <= 0 || D <= 0 || F <= 0 || K <= 0 || ld < D || act < 0 || act >= BN_UNARY_KINDS) return BN_ERR_ARG;
-    if (!h || !w_up || !w_down || !ids || !wts || !y || (size_t)(D + F) * sizeof(float) > 64 * 1024) return BN_ERR_ARG;
+                              const float* wts, float* y, float* hidden, int n_tokens, int y_rows, int D, int F, int K, int act,
+                              int weight_on_input, hipStream_t s) {
+    if (n_tokens <= 0 || y_rows < n_tokens || D <= 0 || F <= 0 || K <= 0 || ld < D || act < 0 || act >= BN_UNARY_KINDS) return BN_ERR_ARG;
+    if (!h || !w_up || !w_down || !ids || !wts || !y || !hidden) return BN_ERR_ARG;
+    if ((size_t)D * sizeof(float) > 64 * 1024 || (size_t)F * sizeof(float) > 64 * 1024 || (size_t)n_tokens * K > 65535) return BN_ERR_ARG;
     PairArgs a;
-    a.h = h; a.w_up = w_up; a.w_down = w_down; a.ids = ids; a.wts = wts; a.y = y;
-    a.ld = ld; a.T = n_tokens; a.D = D; a.F = F; a.K = K; a.act = act; a.weight_on_input = weight_on_input ? 1 : 0;
-    const size_t shm = (size_t)(D + F) * sizeof(float);
-    const dim3 grid((unsigned)n_tokens * K), block(MOE_PAIR_THREADS);
-    if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_pair_kernel<float>, grid, block, shm, s, a);
-    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_pair_kernel<bf16>, grid, block, shm, s, a);
-    else return BN_ERR_DTYPE;
+    a.h = h; a.w_up = w_up; a.w_down = w_down; a.ids = ids; a.wts = wts; a.y = y; a.hidden = hidden;
+    a.ld = ld; a.T = y_rows; a.D = D; a.F = F; a.K = K; a.act = act; a.weight_on_input = weight_on_input ? 1 : 0;
+    const dim3 block(MOE_PAIR_THREADS);
+    const dim3 up((F + MOE_PAIR_ROWS - 1) / MOE_PAIR_ROWS, n_tokens * K), down((D + MOE_PAIR_ROWS - 1) / MOE_PAIR_ROWS, n_tokens * K);
+    if (dtype == BN_DT_F32) {
+        hipLaunchKernelGGL(moe_pair_up_kernel<float>, up, block, (size_t)D * sizeof(float), s, a);
+        hipLaunchKernelGGL(moe_pair_down_kernel<float>, down, block, (size_t)F * sizeof(float), s, a);
+    } else if (dtype == BN_DT_BF16) {
+        hipLaunchKernelGGL(moe_pair_up_kernel<bf16>, up, block, (size_t)D * sizeof(float), s, a);
+        hipLaunchKernelGGL(moe_pair_down_kernel<bf16>, down, block, (size_t)F * sizeof(float), s, a);
+    } else return BN_ERR_DTYPE;
     return bn_launch_status();
 }
 

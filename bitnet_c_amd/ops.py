@@ -67,8 +67,8 @@ _SIGNATURES = {
     "moe": {
         "bn_moe_route": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                          c_void_p],
-        "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                           c_int, c_int, c_void_p],
+        "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                           c_int, c_int, c_int, c_int, c_void_p],
         "bn_moe_grouped_supports": [c_int, c_int],
         "bn_moe_grouped_tiles": [c_int, c_int],
         "bn_moe_grouped": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -1821,12 +1821,17 @@ def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: 
                           f"{tuple(ids.shape)} do not fit")
     if activation not in UNARY_ACTIVATIONS:
         raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
-    if (D + F) * 4 > 65536:
-        raise KernelError(f"moe_experts: width {D} and expert width {F} together are above 16,384 values")
+    if max(D, F) > 16384 or K > 65535:
+        raise KernelError(f"moe_experts: width {D} / expert width {F} above 16,384 values")
     y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
-    if T:
-        _check(_fn("moe", "bn_moe_experts")(_code(h.dtype), h.data_ptr(), _rows(h, "h"), w_up.data_ptr(), w_down.data_ptr(),
-                                            ids.data_ptr(), wts.data_ptr(), y.data_ptr(), T, D, F, K,
+    run = 65535 // K                                      # tokens of one launch: a pair a row of the grid
+    ld = _rows(h, "h")
+    for t0 in range(0, T, run):
+        n = min(run, T - t0)
+        hidden = torch.empty((n * K, F), dtype=torch.float32, device=h.device)
+        _check(_fn("moe", "bn_moe_experts")(_code(h.dtype), h.data_ptr() + t0 * ld * h.element_size(), ld, w_up.data_ptr(),
+                                            w_down.data_ptr(), ids.data_ptr() + t0 * K * 4, wts.data_ptr() + t0 * K * 4,
+                                            y.data_ptr() + t0 * D * 4, hidden.data_ptr(), n, T, D, F, K,
                                             UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)), _stream()), "moe_experts")
     return PartialSums(y)
 

@@ -28,6 +28,11 @@
 // Workgroups are numbered so that the eight XCDs (consecutive workgroup ids go to consecutive
 // XCDs, each with an L2 of its own) each take a band of W and run through all row tiles of X for
 // it: a tile of W comes from HBM once.
+//
+// Grouped form (a mixture of experts): W is a stack of matrices and the rows of X are ordered by the matrix they meet.  A
+// list in device memory cuts the rows into tiles of up to 256 rows of one matrix each (matrix, first row, rows); the grid
+// is laid out for the most tiles there can be and a workgroup whose tile is not in the list leaves.  A row's result may
+// go to another row of Y (row_map), be scaled (row_scale) and pass an activation of one argument first.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -46,6 +51,15 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 gm_as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
+struct GmGroups {
+    const int* tiles;         // [n][3]: matrix of the stack, first row of X, rows (<= GM_BM); null: one product over all rows
+    const int* n_tiles;       // [1]: tiles in the list
+    const int* row_map;       // [rows of X]: the row of Y that takes row m's result; null: m
+    const float* row_scale;   // [rows of X]: a factor on row m's result; null: none
+    long long w_stride;       // elements from one matrix of the stack to the next
+    int unary;                // BN_UNARY_* applied to the result before anything else; < 0: none
+};
+
 // Shared memory serves a 16-byte read in four turns of 16 lanes; in the operand layout
 // (lane = i + 16 g reads chunk c0 + g of row i) a turn holds two values of g and, for each, two
 // values of i / 4.  Two 128-byte rows share the 256 bytes that the banks span: the row's lowest
@@ -58,7 +72,7 @@ __device__ __forceinline__ int gm_swizzle(int row) {
 template <int BN, bool GLU8, typename TO>
 __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W,
                                                                TO* __restrict__ Y, int M, int N, int K, int ldx, int ldw,
-                                                               int ldy, int tiles_m, int tiles_n, int vec, int act) {
+                                                               int ldy, int tiles_m, int tiles_n, int vec, int act, GmGroups grp) {
     constexpr int WM = GM_BM / GM_WGM, WN = BN / GM_WGN;      // a wave's part of the tile
     constexpr int MT = WM / 16, NT = WN / 16;         // 16 x 16 result tiles of a wave: MT x NT
     constexpr int PASS = GM_THREADS / 8;              // rows staged by one pass of the workgroup
@@ -70,7 +84,15 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
     const int xcd = blockIdx.x % GM_XCDS, local = blockIdx.x / GM_XCDS;
     const int tn = xcd + GM_XCDS * (local / tiles_m), tm = local % tiles_m;
     if (tn >= tiles_n) return;                        // the grid is padded to a multiple of 8 column tiles
-    const int m0 = tm * GM_BM, n0 = tn * BN;
+    int m0 = tm * GM_BM;
+    const int n0 = tn * BN;
+    if (grp.tiles) {                                  // the tile's rows end where its matrix's rows end
+        if (tm >= grp.n_tiles[0]) return;
+        const int* tl = grp.tiles + 3 * tm;
+        W += (size_t)tl[0] * grp.w_stride;
+        m0 = tl[1];
+        M = tl[1] + tl[2];
+    }
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int i = lane & 15, g = lane >> 4;
@@ -255,15 +277,27 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_mfma_kernel(const bf16* __res
                     store4(Y + (size_t)m * ldy + f, v, (N >> 1) - f);
                 }
             } else if (m < M) {
-                store4(Y + (size_t)m * ldy + n, v, N - n);
+                if (grp.unary >= 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = bn_unary_act(v[r], grp.unary);
+                }
+                if (grp.row_scale) v *= grp.row_scale[m];
+                const size_t mo = grp.row_map ? (size_t)grp.row_map[m] : (size_t)m;
+                store4(Y + mo * ldy + n, v, N - n);
             }
         }
     }
 }
 
+static GmGroups gm_no_groups() {
+    GmGroups g;
+    g.tiles = nullptr; g.n_tiles = nullptr; g.row_map = nullptr; g.row_scale = nullptr; g.w_stride = 0; g.unary = -1;
+    return g;
+}
+
 template <int BN, bool GLU8, typename TO>
 static int gm_launch(const void* X, const void* W, void* Y, int M, int N, int K, int ldx, int ldw, int ldy, int act,
-                     hipStream_t s) {
+                     hipStream_t s, GmGroups grp = gm_no_groups(), int max_tiles = 0) {
     auto kernel = gemm_mfma_kernel<BN, GLU8, TO>;
     const size_t smem = (size_t)2 * (GM_BM + BN) * 128;
     static bool raised = false;                       // per instantiation
@@ -273,13 +307,13 @@ static int gm_launch(const void* X, const void* W, void* Y, int M, int N, int K,
         if (e != hipSuccess) return (int)e;
         raised = true;
     }
-    const int tiles_m = (M + GM_BM - 1) / GM_BM, tiles_n = (N + BN - 1) / BN;
+    const int tiles_m = grp.tiles ? max_tiles : (M + GM_BM - 1) / GM_BM, tiles_n = (N + BN - 1) / BN;
     const int bands = (tiles_n + GM_XCDS - 1) / GM_XCDS;           // column tiles per XCD
     const long long grid = (long long)bands * GM_XCDS * tiles_m;
     if (grid > 0x7fffffffLL) return BN_ERR_ARG;
     const int vec = (ldy % 4 == 0 && ((uintptr_t)Y % (4 * sizeof(TO))) == 0) ? 1 : 0;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(GM_THREADS), smem, s, (const bf16*)X, (const bf16*)W, (TO*)Y,
-                       M, N, K, ldx, ldw, ldy, tiles_m, tiles_n, vec, act);
+                       M, N, K, ldx, ldw, ldy, tiles_m, tiles_n, vec, act, grp);
     return bn_launch_status();
 }
 
@@ -343,4 +377,27 @@ extern "C" int bn_gemm_mfma(int out_dtype, const void* X, const void* W, void* Y
     if (bn == 192) { GM_GO(192, false); }
     GM_GO(128, false);
 #undef GM_GO
+}
+
+// The grouped form: X [rows, K] ordered by matrix, W [matrices][N, K] (w_stride elements apart), tiles [max_tiles][3] and
+// n_tiles [1] in device memory (tiles of at most 256 rows), Y row row_map[m] (or m) = unary(X[m] . W[matrix]^T) * row_scale[m].
+// rows: all rows of X (sizes the tile width).  out_dtype: type of Y.
+extern "C" int bn_gemm_mfma_grouped(int out_dtype, const void* X, const void* W, void* Y, const int* tiles, const int* n_tiles,
+                                    int max_tiles, const int* row_map, const float* row_scale, long long w_stride, int unary,
+                                    int rows, int N, int K, int ldx, int ldw, int ldy, hipStream_t s) {
+    if (!bn_gemm_mfma_supports(rows, N, K, ldx, ldw) || ldy < N || max_tiles < 1 || !tiles || !n_tiles || w_stride < 0) return BN_ERR_ARG;
+    if (unary >= BN_UNARY_KINDS || (((uintptr_t)X | (uintptr_t)W) & 15) || (w_stride % 8)) return BN_ERR_ARG;
+    if (out_dtype != BN_DT_BF16 && out_dtype != BN_DT_F32) return BN_ERR_DTYPE;
+    GmGroups g;
+    g.tiles = tiles; g.n_tiles = n_tiles; g.row_map = row_map; g.row_scale = row_scale; g.w_stride = w_stride;
+    g.unary = unary < 0 ? -1 : unary;
+    const int bn = gm_pick_bn(rows, N, gm_compute_units());
+    const bool f32 = out_dtype == BN_DT_F32;
+#define GM_GROUPED(BN_)                                                                                         \
+    return f32 ? gm_launch<BN_, false, float>(X, W, Y, rows, N, K, ldx, ldw, ldy, 0, s, g, max_tiles)          \
+               : gm_launch<BN_, false, bf16>(X, W, Y, rows, N, K, ldx, ldw, ldy, 0, s, g, max_tiles)
+    if (bn == 256) { GM_GROUPED(256); }
+    if (bn == 192) { GM_GROUPED(192); }
+    GM_GROUPED(128);
+#undef GM_GROUPED
 }

@@ -61,7 +61,8 @@ extern "C" int bn_latent_store(int dtype, const void* x, int ld, int col, const 
 
 // ---- a product per head ---------------------------------------------------------------------------------------------
 #define HL_ROWS 8             // rows of x that a workgroup takes
-#define HL_COLS 128           // output columns of a workgroup: one a thread
+#define HL_COLS 64            // output columns of a workgroup
+#define HL_SLICES 4           // parts of the input dimension, a wave each; their sums meet in shared memory
 
 struct HeadLinearArgs {
     const void* x;            // [T, ldx]: head h at h * I
@@ -71,35 +72,47 @@ struct HeadLinearArgs {
     int ldx, ldy, ldg, T, H, I, O;
 };
 
-// The rows of x are staged in shared memory as float32 and read by every thread at the same address; a thread walks the
-// input dimension with one coalesced load of the weights a step.
+// The rows of x are staged in shared memory as float32 and read by every lane of a wave at the same address; a lane owns
+// an output column and walks its wave's part of the input dimension with one coalesced load of the weights a step, eight
+// steps' loads in flight.
 template <typename T>
-__global__ __launch_bounds__(HL_COLS) void head_linear_kernel(HeadLinearArgs a) {
-    extern __shared__ float xs[];                        // [HL_ROWS][I]
-    const int h = blockIdx.y, t0 = blockIdx.z * HL_ROWS, o = blockIdx.x * HL_COLS + threadIdx.x;
+__global__ __launch_bounds__(HL_COLS * HL_SLICES) void head_linear_kernel(HeadLinearArgs a) {
+    extern __shared__ float xs[];                        // [HL_ROWS][I], then the slices' sums [HL_SLICES][HL_ROWS][HL_COLS]
+    float* red = xs + HL_ROWS * a.I;
+    const int h = blockIdx.y, t0 = blockIdx.z * HL_ROWS, c = threadIdx.x & (HL_COLS - 1), slice = threadIdx.x / HL_COLS;
+    const int o = blockIdx.x * HL_COLS + c;
     const int rows = min(HL_ROWS, a.T - t0);
     const T* x = reinterpret_cast<const T*>(a.x);
-    for (int idx = threadIdx.x; idx < HL_ROWS * a.I; idx += HL_COLS) {
+    for (int idx = threadIdx.x; idx < HL_ROWS * a.I; idx += HL_COLS * HL_SLICES) {
         const int r = idx / a.I, i = idx - r * a.I;
         xs[idx] = r < rows ? to_f32(x[(size_t)(t0 + r) * a.ldx + (size_t)h * a.I + i]) : 0.f;
     }
     __syncthreads();
-    if (o >= a.O) return;
     float acc[HL_ROWS];
 #pragma unroll
     for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
-    const T* w = reinterpret_cast<const T*>(a.w) + (size_t)h * a.I * a.O + o;
-    for (int i = 0; i < a.I; ++i) {
-        const float wv = to_f32(w[(size_t)i * a.O]);
+    const int per = (a.I + HL_SLICES - 1) / HL_SLICES, i0 = slice * per, i1 = min(a.I, i0 + per);
+    if (o < a.O) {
+        const T* w = reinterpret_cast<const T*>(a.w) + (size_t)h * a.I * a.O + o;
+#pragma unroll 8
+        for (int i = i0; i < i1; ++i) {
+            const float wv = to_f32(w[(size_t)i * a.O]);
 #pragma unroll
-        for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(xs[r * a.I + i], wv, acc[r]);
+            for (int r = 0; r < HL_ROWS; ++r) acc[r] = fmaf(xs[r * a.I + i], wv, acc[r]);
+        }
     }
+#pragma unroll
+    for (int r = 0; r < HL_ROWS; ++r) red[(slice * HL_ROWS + r) * HL_COLS + c] = acc[r];
+    __syncthreads();
+    if (slice != 0 || o >= a.O) return;
     T* y = reinterpret_cast<T*>(a.y);
     const T* g = reinterpret_cast<const T*>(a.gate);
 #pragma unroll
     for (int r = 0; r < HL_ROWS; ++r) {
         if (r >= rows) break;
-        float v = acc[r];
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < HL_SLICES; ++k) v += red[(k * HL_ROWS + r) * HL_COLS + c];
         if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + (size_t)h * a.O + o])));
         y[(size_t)(t0 + r) * a.ldy + (size_t)h * a.O + o] = from_f32<T>(v);
     }
@@ -108,13 +121,13 @@ __global__ __launch_bounds__(HL_COLS) void head_linear_kernel(HeadLinearArgs a) 
 extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, void* y, int ldy, const void* gate, int ldg,
                               int n_rows, int H, int I, int O, hipStream_t s) {
     if (n_rows <= 0 || H <= 0 || I <= 0 || O <= 0 || !x || !w || !y) return BN_ERR_ARG;
-    if (ldx < H * I || ldy < H * O || (gate && ldg < H * O) || (size_t)HL_ROWS * I * sizeof(float) > 64 * 1024 || H > 65535) return BN_ERR_ARG;
+    if (ldx < H * I || ldy < H * O || (gate && ldg < H * O) || (size_t)HL_ROWS * (I + HL_SLICES * HL_COLS) * sizeof(float) > 64 * 1024 || H > 65535) return BN_ERR_ARG;
     const int row_tiles = (n_rows + HL_ROWS - 1) / HL_ROWS;
     if (row_tiles > 65535) return BN_ERR_ARG;
     HeadLinearArgs a;
     a.x = x; a.w = w; a.y = y; a.gate = gate; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.T = n_rows; a.H = H; a.I = I; a.O = O;
-    const dim3 grid((O + HL_COLS - 1) / HL_COLS, H, row_tiles), block(HL_COLS);
-    const size_t shm = (size_t)HL_ROWS * I * sizeof(float);
+    const dim3 grid((O + HL_COLS - 1) / HL_COLS, H, row_tiles), block(HL_COLS * HL_SLICES);
+    const size_t shm = (size_t)HL_ROWS * (I + HL_SLICES * HL_COLS) * sizeof(float);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(head_linear_kernel<float>, grid, block, shm, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(head_linear_kernel<bf16>, grid, block, shm, s, a);
     else return BN_ERR_DTYPE;

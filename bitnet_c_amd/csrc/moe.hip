@@ -1,14 +1,14 @@
 // A mixture-of-experts feed-forward whose experts have no gate: expert e is  W_down[e] act(W_up[e] x).
 //
-//   bn_moe_route     router logits z = W_r h in float32 (one wave a token), scores sigmoid(z) or softmax(z), the top_k
+//   bn_moe_route     router logits z = W_r h in float32 (one workgroup a token), scores sigmoid(z) or softmax(z), the top_k
 //                    largest (ties: the lower index), optionally divided by their sum -> expert ids and weights [T, top_k]
 //   bn_moe_experts   for every (token, choice) pair: y = W_down[e] act(W_up[e] (w h)) when the weight multiplies the
 //                    expert's input, w * W_down[e] act(W_up[e] h) when it multiplies the output; a pair reads its expert's
 //                    two matrices once, their rows spread over workgroups.  The products accumulate in float32; the scaled
 //                    input and the hidden vector are rounded to the activations' type as a product of that type would
 //                    see them.
-//   bn_moe_plan      pairs ordered by expert, and tiles of up to MOE_TILE rows of one expert each, for the grouped products
-//   bn_moe_grouped   (bf16) the same two products on the matrix cores over those tiles: a tile's rows share an expert
+//   bn_moe_group     (bf16, steps of many rows) pairs ordered by expert, tiles of rows of one expert each, and the inputs
+//                    gathered in that order, for the grouped matrix products of gemm_mfma.hip
 // The outputs of a token's choices land in slab j of y [top_k, T, D] (float32) and are added by whoever consumes y.
 #include "common.h"
 #include <math.h>
@@ -26,25 +26,38 @@ struct RouteArgs {
     int ld, D, E, K, scoring, renorm;
 };
 
+#define MOE_ROUTE_THREADS 256
+
+// One workgroup a token: its waves take the experts in turn (a row of the router as 16-byte loads across the lanes, several
+// in flight), the first wave then chooses.
 template <typename T>
-__global__ __launch_bounds__(BN_WAVE) void moe_route_kernel(RouteArgs a) {
-    extern __shared__ float hs[];                        // the token's row as float32
-    const int t = blockIdx.x, lane = threadIdx.x;
+__global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs a) {
+    extern __shared__ __align__(16) float hs[];          // the token's row as float32, then the experts' logits
+    float* zs = hs + ((a.D + 3) & ~3);
+    const int t = blockIdx.x, lane = threadIdx.x & (BN_WAVE - 1), wave = threadIdx.x / BN_WAVE;
     const T* h = reinterpret_cast<const T*>(a.h) + (size_t)t * a.ld;
-    for (int d = lane; d < a.D; d += BN_WAVE) hs[d] = to_f32(h[d]);
+    for (int d = threadIdx.x; d < a.D; d += MOE_ROUTE_THREADS) hs[d] = to_f32(h[d]);
     __syncthreads();
-    float z[MOE_PER_LANE];                               // expert lane + 64 j
-#pragma unroll
-    for (int j = 0; j < MOE_PER_LANE; ++j) z[j] = -INFINITY;
-    for (int e = 0; e < a.E; ++e) {
+    for (int e = wave; e < a.E; e += MOE_ROUTE_THREADS / BN_WAVE) {
         const float* w = a.wr + (size_t)e * a.D;
         float s = 0.f;
-        for (int d = lane; d < a.D; d += BN_WAVE) s = fmaf(hs[d], w[d], s);
+        if (a.D % 4 == 0) {
+#pragma unroll 4
+            for (int d = 4 * lane; d < a.D; d += 4 * BN_WAVE) {
+                const float4 wv = *reinterpret_cast<const float4*>(w + d), xv = *reinterpret_cast<const float4*>(hs + d);
+                s = fmaf(xv.x, wv.x, s); s = fmaf(xv.y, wv.y, s); s = fmaf(xv.z, wv.z, s); s = fmaf(xv.w, wv.w, s);
+            }
+        } else {
+            for (int d = lane; d < a.D; d += BN_WAVE) s = fmaf(hs[d], w[d], s);
+        }
         s = wave_sum(s);
-#pragma unroll
-        for (int j = 0; j < MOE_PER_LANE; ++j)
-            if (e == lane + BN_WAVE * j) z[j] = s;
+        if (lane == 0) zs[e] = s;
     }
+    __syncthreads();
+    if (wave != 0) return;
+    float z[MOE_PER_LANE];                               // expert lane + 64 j
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j) z[j] = lane + BN_WAVE * j < a.E ? zs[lane + BN_WAVE * j] : -INFINITY;
     float zmax = -INFINITY, denom = 1.f;
     if (a.scoring == MOE_SCORE_SOFTMAX) {
 #pragma unroll
@@ -95,12 +108,12 @@ extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, i
     if (n_tokens <= 0 || D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || K <= 0 || K > E || ld < D || !h || !wr || !ids || !wts)
         return BN_ERR_ARG;
     if (scoring != MOE_SCORE_SIGMOID && scoring != MOE_SCORE_SOFTMAX) return BN_ERR_ARG;
-    if ((size_t)D * sizeof(float) > 64 * 1024) return BN_ERR_ARG;
+    if ((size_t)(D + 4 + E) * sizeof(float) > 64 * 1024 || ((uintptr_t)wr & 15)) return BN_ERR_ARG;
     RouteArgs a;
     a.h = h; a.wr = wr; a.ids = ids; a.wts = wts; a.ld = ld; a.D = D; a.E = E; a.K = K; a.scoring = scoring; a.renorm = renorm ? 1 : 0;
-    const size_t shm = (size_t)D * sizeof(float);
-    if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(BN_WAVE), shm, s, a);
-    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(BN_WAVE), shm, s, a);
+    const size_t shm = (size_t)(((D + 3) & ~3) + E) * sizeof(float);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);
     else return BN_ERR_DTYPE;
     return bn_launch_status();
 }
@@ -111,7 +124,7 @@ extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, i
 // the pair's input vector in shared memory as float32, each of its waves takes MOE_PAIR_ROWS / 4 rows of the matrix, a row
 // as 16-byte loads across the lanes (bf16 rows of whole 8-element groups) or element by element, and sums in float32.
 #define MOE_PAIR_THREADS 256
-#define MOE_PAIR_ROWS 16
+#define MOE_PAIR_ROWS 8
 
 struct PairArgs {
     const void* h;            // [T, ld]
@@ -210,21 +223,15 @@ extern "C" int bn_moe_experts(int dtype, const void* h, int ld, const void* w_up
     return bn_launch_status();
 }
 
-// ---- grouped products on the matrix cores (bf16) ---------------------------------------------------------------------
-// The pairs of a step are ordered by expert and cut into tiles of up to MOE_TILE rows of one expert; a workgroup takes one
-// tile and 64 columns of the product, its four waves 16 columns each: a wave loads a 16 x 32 piece of the expert's matrix
-// once and uses it for both 16-row halves of the tile (v_mfma_f32_16x16x32_bf16; the matrix as the first operand, so that
-// a lane ends up with four consecutive result columns of one row: one store).  Operands come straight from memory, 16 bytes
-// a lane; everything that a tile needs to know lies in device memory, so the launches do not depend on the routing.
-#define MOE_TILE 32
+// ---- steps of many rows: pairs ordered by expert (bf16) ---------------------------------------------------------------
+// The pairs of a step are ordered by expert and cut into tiles of up to tile_rows rows of one expert; the inputs are
+// gathered in that order (scaled by the pair's weight and rounded, when the weight multiplies the input), and the two
+// products run as grouped matrix products over the tiles (gemm_mfma.hip).  Everything a tile needs to know lies in device
+// memory, so the launches do not depend on the routing.
 #define MOE_PLAN_THREADS 1024
 
-typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
-typedef __attribute__((ext_vector_type(8))) float moe_f32x8;
-typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
-
 // order [T K]: the pairs (t K + j) by expert; tiles [max_tiles][3] = expert, first place in `order`, rows; n_tiles [1]
-__global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* __restrict__ ids, int n_pairs, int E,
+__global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* __restrict__ ids, int n_pairs, int E, int tile_rows,
                                                                     int* __restrict__ order, int* __restrict__ tiles,
                                                                     int* __restrict__ n_tiles) {
     __shared__ int count[MOE_MAX_EXPERTS], first[MOE_MAX_EXPERTS + 1], tile0[MOE_MAX_EXPERTS + 1];
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* _
         for (int e = 0; e < E; ++e) {
             first[e] = at; tile0[e] = tl;
             at += count[e];
-            tl += (count[e] + MOE_TILE - 1) / MOE_TILE;
+            tl += (count[e] + tile_rows - 1) / tile_rows;
         }
         first[E] = at; tile0[E] = tl;
         n_tiles[0] = tl;
@@ -245,8 +252,8 @@ __global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* _
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         const int n = count[e];
-        for (int r = 0, k = tile0[e]; r < n; r += MOE_TILE, ++k) {
-            tiles[3 * k] = e; tiles[3 * k + 1] = first[e] + r; tiles[3 * k + 2] = min(MOE_TILE, n - r);
+        for (int r = 0, k = tile0[e]; r < n; r += tile_rows, ++k) {
+            tiles[3 * k] = e; tiles[3 * k + 1] = first[e] + r; tiles[3 * k + 2] = min(tile_rows, n - r);
         }
         count[e] = 0;                                    // now the cursor of the scatter
     }
@@ -259,122 +266,47 @@ __global__ __launch_bounds__(MOE_PLAN_THREADS) void moe_plan_kernel(const int* _
     }
 }
 
-struct GroupedArgs {
-    const bf16* x;            // up: h [T, ldx]; down: hidden [pairs, F] in the order of `order`
-    const bf16* w;            // up: [E, F, D]; down: [E, D, F]
-    bf16* hidden;             // up's result
-    float* y;                 // down's result [K, T, D]
-    const int* order;
-    const int* tiles;
-    const int* n_tiles;
-    const float* wts;         // [T, K]
-    int ldx, T, D, F, K, act, weight_on_input;
-};
-
-__device__ __forceinline__ moe_bf16x8 moe_ld16(const bf16* p) {
-    return __builtin_bit_cast(moe_bf16x8, *reinterpret_cast<const uint4*>(p));
-}
-
-// hidden[place] = act(W_up[e] (w h[t]))  for the rows of a tile; N = F columns, the sum runs over D
-__global__ __launch_bounds__(256) void moe_grouped_up_kernel(GroupedArgs a) {
-    const int tile = blockIdx.x;
-    if (tile >= a.n_tiles[0]) return;
-    const int e = a.tiles[3 * tile], start = a.tiles[3 * tile + 1], rows = a.tiles[3 * tile + 2];
-    const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
-    const int f0 = blockIdx.y * 64 + 16 * (threadIdx.x >> 6);
-    if (f0 >= a.F) return;
-    const bf16* wrow = a.w + ((size_t)e * a.F + f0 + i) * a.D + 8 * g;
-    const bf16* xrow[2];
-    float sc[2];
+// xg[place] = h[token of the pair at that place] (times the pair's weight, rounded to bf16, when scale_input); row_map[place]
+// = the pair's row of y seen as [K T, D]; row_scale[place] = the pair's weight.  One workgroup a place, 16 bytes a thread.
+__global__ __launch_bounds__(256) void moe_gather_kernel(const bf16* __restrict__ h, int ld, const int* __restrict__ order,
+                                                         const float* __restrict__ wts, bf16* __restrict__ xg,
+                                                         int* __restrict__ row_map, float* __restrict__ row_scale, int T, int D,
+                                                         int K, int scale_input) {
+    const int place = blockIdx.x, pair = order[place], t = pair / K, j = pair - t * K;
+    const float w = wts[pair];
+    if (threadIdx.x == 0) { row_map[place] = j * T + t; row_scale[place] = w; }
+    const bf16* src = h + (size_t)t * ld;
+    bf16* dst = xg + (size_t)place * D;
+    for (int d = 8 * threadIdx.x; d < D; d += 8 * 256) {
+        uint4 p = *reinterpret_cast<const uint4*>(src + d);
+        if (scale_input) {
+            uint32_t* q = reinterpret_cast<uint32_t*>(&p);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        const int pair = a.order[start + min(16 * s + i, rows - 1)];
-        xrow[s] = a.x + (size_t)(pair / a.K) * a.ldx + 8 * g;
-        sc[s] = a.weight_on_input ? a.wts[pair] : 1.0f;
-    }
-    moe_f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    for (int c = 0; c < a.D; c += 32) {
-        const moe_bf16x8 wf = moe_ld16(wrow + c);
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            if (s == 1 && rows <= 16) break;
-            moe_bf16x8 xf = moe_ld16(xrow[s] + c);
-            if (a.weight_on_input) {                     // the expert reads w h, rounded to the activations' type
-                moe_f32x8 xv = __builtin_convertvector(xf, moe_f32x8);
-                xv *= sc[s];
-                xf = __builtin_convertvector(xv, moe_bf16x8);
+            for (int k = 0; k < 4; ++k) {
+                const bf16 lo = __float2bfloat16(bf16lo_to_f32(q[k]) * w), hi = __float2bfloat16(bf16hi_to_f32(q[k]) * w);
+                q[k] = (uint32_t)__builtin_bit_cast(unsigned short, lo) | ((uint32_t)__builtin_bit_cast(unsigned short, hi) << 16);
             }
-            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[s], 0, 0, 0);
         }
-    }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        const int r = 16 * s + i;
-        if (r >= rows) continue;
-        bf16 o[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = __float2bfloat16(bn_unary_act(acc[s][k], a.act));
-        uint2 pk;
-        pk.x = (uint32_t)__builtin_bit_cast(unsigned short, o[0]) | ((uint32_t)__builtin_bit_cast(unsigned short, o[1]) << 16);
-        pk.y = (uint32_t)__builtin_bit_cast(unsigned short, o[2]) | ((uint32_t)__builtin_bit_cast(unsigned short, o[3]) << 16);
-        *reinterpret_cast<uint2*>(a.hidden + (size_t)(start + r) * a.F + f0 + 4 * g) = pk;
+        *reinterpret_cast<uint4*>(dst + d) = p;
     }
 }
 
-// y[j][t] = W_down[e] hidden[place] (times w when the weight multiplies the output); N = D columns, the sum runs over F
-__global__ __launch_bounds__(256) void moe_grouped_down_kernel(GroupedArgs a) {
-    const int tile = blockIdx.x;
-    if (tile >= a.n_tiles[0]) return;
-    const int e = a.tiles[3 * tile], start = a.tiles[3 * tile + 1], rows = a.tiles[3 * tile + 2];
-    const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
-    const int d0 = blockIdx.y * 64 + 16 * (threadIdx.x >> 6);
-    if (d0 >= a.D) return;
-    const bf16* wrow = a.w + ((size_t)e * a.D + d0 + i) * a.F + 8 * g;
-    const bf16* xrow[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) xrow[s] = a.x + (size_t)(start + min(16 * s + i, rows - 1)) * a.F + 8 * g;
-    moe_f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    for (int c = 0; c < a.F; c += 32) {
-        const moe_bf16x8 wf = moe_ld16(wrow + c);
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            if (s == 1 && rows <= 16) break;
-            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, moe_ld16(xrow[s] + c), acc[s], 0, 0, 0);
-        }
-    }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        const int r = 16 * s + i;
-        if (r >= rows) continue;
-        const int pair = a.order[start + r], t = pair / a.K, j = pair - t * a.K;
-        const float f = a.weight_on_input ? 1.0f : a.wts[pair];
-        float4 o = make_float4(acc[s][0] * f, acc[s][1] * f, acc[s][2] * f, acc[s][3] * f);
-        *reinterpret_cast<float4*>(a.y + ((size_t)j * a.T + t) * a.D + d0 + 4 * g) = o;
-    }
+extern "C" int bn_moe_grouped_tiles(int n_pairs, int E, int tile_rows) {
+    return tile_rows > 0 ? (n_pairs + tile_rows - 1) / tile_rows + E : 0;
 }
 
-// 1 if the grouped products take these sizes (the sums run over whole chunks of 32, the columns come in sixteens)
-extern "C" int bn_moe_grouped_supports(int D, int F) { return (D > 0 && F > 0 && D % 32 == 0 && F % 32 == 0) ? 1 : 0; }
-extern "C" int bn_moe_grouped_tiles(int n_pairs, int E) { return (n_pairs + MOE_TILE - 1) / MOE_TILE + E; }
-
-// work: int32 [n_pairs + 3 max_tiles + 1] (order, tiles, n_tiles); hidden: bf16 [n_pairs, F]
-extern "C" int bn_moe_grouped(const void* h, int ld, const void* w_up, const void* w_down, const int* ids, const float* wts,
-                              float* y, int* work, void* hidden, int n_tokens, int D, int F, int E, int K, int act,
-                              int weight_on_input, hipStream_t s) {
-    if (n_tokens <= 0 || K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || !bn_moe_grouped_supports(D, F) || ld < D || ld % 8) return BN_ERR_ARG;
-    if (act < 0 || act >= BN_UNARY_KINDS || !h || !w_up || !w_down || !ids || !wts || !y || !work || !hidden) return BN_ERR_ARG;
-    if ((((uintptr_t)h | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)y | (uintptr_t)hidden) & 15)) return BN_ERR_ARG;
-    const int n_pairs = n_tokens * K, max_tiles = bn_moe_grouped_tiles(n_pairs, E);
+// work: int32 [2 n_pairs + 3 max_tiles + 1] = order, row_map, tiles, n_tiles; row_scale: float32 [n_pairs]; xg: bf16 [n_pairs, D]
+extern "C" int bn_moe_group(const void* h, int ld, const int* ids, const float* wts, int* work, float* row_scale, void* xg,
+                            int n_tokens, int D, int E, int K, int tile_rows, int scale_input, hipStream_t s) {
+    if (n_tokens <= 0 || K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || D <= 0 || D % 8 || ld < D || ld % 8 || tile_rows <= 0) return BN_ERR_ARG;
+    if (!h || !ids || !wts || !work || !row_scale || !xg || (((uintptr_t)h | (uintptr_t)xg) & 15)) return BN_ERR_ARG;
+    const int n_pairs = n_tokens * K, max_tiles = bn_moe_grouped_tiles(n_pairs, E, tile_rows);
     int* order = work;
-    int* tiles = work + n_pairs;
+    int* row_map = work + n_pairs;
+    int* tiles = row_map + n_pairs;
     int* n_tiles = tiles + 3 * max_tiles;
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(MOE_PLAN_THREADS), 0, s, ids, n_pairs, E, order, tiles, n_tiles);
-    GroupedArgs a;
-    a.x = (const bf16*)h; a.w = (const bf16*)w_up; a.hidden = (bf16*)hidden; a.y = y; a.order = order; a.tiles = tiles;
-    a.n_tiles = n_tiles; a.wts = wts; a.ldx = ld; a.T = n_tokens; a.D = D; a.F = F; a.K = K; a.act = act;
-    a.weight_on_input = weight_on_input ? 1 : 0;
-    hipLaunchKernelGGL(moe_grouped_up_kernel, dim3(max_tiles, (F + 63) / 64), dim3(256), 0, s, a);
-    a.x = (const bf16*)hidden; a.w = (const bf16*)w_down;
-    hipLaunchKernelGGL(moe_grouped_down_kernel, dim3(max_tiles, (D + 63) / 64), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(MOE_PLAN_THREADS), 0, s, ids, n_pairs, E, tile_rows, order, tiles, n_tiles);
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(n_pairs), dim3(256), 0, s, (const bf16*)h, ld, order, wts, (bf16*)xg, row_map,
+                       row_scale, n_tokens, D, K, scale_input ? 1 : 0);
     return bn_launch_status();
 }

@@ -36,7 +36,18 @@ struct QkNormArgs {
     int temp_every;           // <= 0: no temperature
 };
 
-// one workgroup per row, its waves take the heads in turn; heads 0 .. H-1 are queries, then Hkv keys, then Hkv values
+// sine and cosine of an angle of any size: the angle less the nearest multiple of 2 pi (2 pi as the sum of two floats, the
+// products exact inside the fused operations), then the hardware's functions on what is left, which lies in [-pi, pi]
+__device__ __forceinline__ void qkn_sincos(float a, float* sn, float* cs) {
+    const float k = rintf(a * 0.15915494309189535f);
+    float r = fmaf(-k, 6.2831854820251465f, a);
+    r = fmaf(-k, -1.7484555e-7f, r);
+    *sn = __sinf(r);
+    *cs = __cosf(r);
+}
+
+// a workgroup takes QKN_WAVES heads of one row, a wave each; heads 0 .. H-1 are queries, then Hkv keys, then Hkv values.
+// With norms over the whole projections every workgroup of a row forms the two sums of squares for itself.
 template <typename T>
 __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNormArgs a) {
     __shared__ float scratch[16];
@@ -56,7 +67,7 @@ __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNo
         fk = 1.0f / sqrtf(sk / (float)nk + a.eps);
     }
     const int rd = a.inv_freq ? a.rope_dims : 0, half = rd / 2;
-    for (int head = wave; head < a.H + 2 * a.Hkv; head += QKN_WAVES) {
+    for (int head = blockIdx.y * QKN_WAVES + wave; head < min(a.H + 2 * a.Hkv, (int)(blockIdx.y + 1) * QKN_WAVES); head += QKN_WAVES) {
         const bool is_q = head < a.H, is_k = !is_q && head < a.H + a.Hkv;
         if (is_q || is_k) {
             if (is_k && !a.k_pages) continue;
@@ -103,7 +114,7 @@ __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNo
                     const int i = a.rope_interleaved ? (d >> 1) : (d < half ? d : d - half);
                     const bool first = a.rope_interleaved ? !(d & 1) : d < half;
                     float sn, cs;
-                    sincosf((float)pos * a.inv_freq[i], &sn, &cs);
+                    qkn_sincos((float)pos * a.inv_freq[i], &sn, &cs);
                     x = first ? x * cs - ps[j] * sn : x * cs + ps[j] * sn;
                 }
                 dst[d] = from_f32<T>(x * temp);
@@ -139,7 +150,7 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
     a.ld = ld; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv; a.hs = hs; a.vd = vd;
     a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every; a.v_transposed = v_transposed ? 1 : 0;
     a.norm_all = norm_all ? 1 : 0; a.rope_dims = inv_freq ? rope_dims : 0; a.rope_interleaved = rope_interleaved ? 1 : 0;
-    const dim3 grid(n_tokens), block(QKN_WAVES * BN_WAVE);
+    const dim3 grid(n_tokens, (H + 2 * Hkv + QKN_WAVES - 1) / QKN_WAVES), block(QKN_WAVES * BN_WAVE);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, block, 0, s, a);
     else return BN_ERR_DTYPE;

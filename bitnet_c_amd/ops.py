@@ -69,10 +69,9 @@ _SIGNATURES = {
                          c_void_p],
         "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, c_void_p],
-        "bn_moe_grouped_supports": [c_int, c_int],
-        "bn_moe_grouped_tiles": [c_int, c_int],
-        "bn_moe_grouped": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_moe_grouped_tiles": [c_int, c_int, c_int],
+        "bn_moe_group": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_void_p],
     },
     "attn_mfma_general": {
         "bn_attn_general_supports": [c_int, c_int],
@@ -123,6 +122,8 @@ _SIGNATURES = {
         "bn_gemm_mfma_supports": [c_int, c_int, c_int, c_int, c_int],
         "bn_gemm_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_void_p],
+        "bn_gemm_mfma_grouped": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_longlong,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "skinny_gemm": {
         "bn_skinny_gemm_supports": [c_int, c_int, c_int, c_int, c_int],
@@ -1732,7 +1733,7 @@ def latent_store(x: torch.Tensor, col: int, rank: int, weight: torch.Tensor, eps
                                             _stream()), "latent_store")
 
 
-HEAD_LINEAR_MAX_IN = 2048          # the kernel stages 8 rows of a head's input as float32 in 64 KB of shared memory
+HEAD_LINEAR_MAX_IN = 1792          # the kernel stages 8 rows of a head's input as float32 beside its partial sums in 64 KB of shared memory
 
 
 def head_linear(x: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] = None, *,
@@ -1836,22 +1837,23 @@ def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: 
     return PartialSums(y)
 
 
-MOE_GROUPED_MIN_ROWS = 17           # rows from which a bf16 step's experts run as grouped products (below: a pair a workgroup)
-MOE_TILE = _build.header_constant("MOE_TILE", "moe.hip")
+MOE_GROUPED_MIN_ROWS = 17           # rows from which a bf16 step's experts run as grouped products (below: a pair at a time)
+MOE_TILE_ROWS = _build.header_constant("GM_BM", "gemm_mfma.hip")     # rows of a tile of the grouped products
 
 
 def moe_grouped_supported(T: int, D: int, F: int, dtype) -> bool:
-    """Whether moe_experts_grouped takes a step of T rows of these sizes and is the faster of the two: bf16, sums over whole
-    chunks of 32 (bn_moe_grouped_supports, answered here so that asking loads no kernel), and enough rows for experts to
-    be shared."""
-    return dtype == torch.bfloat16 and T >= MOE_GROUPED_MIN_ROWS and D % 32 == 0 and F % 32 == 0
+    """Whether moe_experts_grouped takes a step of T rows of these sizes and is the faster of the two: bf16, rows of whole
+    16-byte groups, and enough rows for experts to be shared."""
+    return dtype == torch.bfloat16 and T >= MOE_GROUPED_MIN_ROWS and D % 8 == 0 and F % 8 == 0
 
 
 def moe_experts_grouped(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
                         activation: str = "relu2", weight_on_input: bool = True) -> PartialSums:
     """What moe_experts computes, for bf16 steps of many rows: the (token, choice) pairs are ordered by expert on the
-    device and cut into tiles of up to MOE_TILE rows of one expert, and both products run on the matrix cores over those
-    tiles.  Nothing comes back to the host; the launches' sizes depend on the step's shape alone."""
+    device and cut into tiles of up to MOE_TILE_ROWS rows of one expert, the inputs are gathered in that order (scaled
+    and rounded there when the weight multiplies the input), and both products run as grouped matrix products on the matrix
+    cores (the tiled kernel of gemm_mfma with a list of tiles).  Nothing comes back to the host; the launches' sizes depend
+    on the step's shape alone."""
     require_gpu()
     _dev(h, "h", torch.bfloat16, 2)
     _dev(w_up, "w_up", torch.bfloat16, 3)
@@ -1868,19 +1870,29 @@ def moe_experts_grouped(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tenso
     if activation not in UNARY_ACTIVATIONS:
         raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
     ld = _rows(h, "h")
-    if D % 32 or F % 32 or E > MOE_MAX_EXPERTS or ld % 8 or h.data_ptr() % 16:
-        raise KernelError(f"moe_experts_grouped: widths {D} and {F} must be multiples of 32, rows 16-byte aligned, at most "
+    if D % 8 or F % 8 or E > MOE_MAX_EXPERTS or ld % 8 or (h.data_ptr() | w_up.data_ptr() | w_down.data_ptr()) % 16:
+        raise KernelError(f"moe_experts_grouped: widths {D} and {F} must be multiples of 8, rows 16-byte aligned, at most "
                           f"{MOE_MAX_EXPERTS} experts")
     y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
     if T == 0:
         return PartialSums(y)
-    max_tiles = -(-T * K // MOE_TILE) + E
-    work = torch.empty((T * K + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
-    hidden = torch.empty((T * K, F), dtype=torch.bfloat16, device=h.device)
-    _check(_fn("moe", "bn_moe_grouped")(h.data_ptr(), ld, w_up.data_ptr(), w_down.data_ptr(), ids.data_ptr(), wts.data_ptr(),
-                                        y.data_ptr(), work.data_ptr(), hidden.data_ptr(), T, D, F, E, K,
-                                        UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)), _stream()),
-           "moe_experts_grouped")
+    n = T * K
+    max_tiles = -(-n // MOE_TILE_ROWS) + E
+    work = torch.empty((2 * n + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+    row_scale = torch.empty((n,), dtype=torch.float32, device=h.device)
+    xg = torch.empty((n, D), dtype=torch.bfloat16, device=h.device)
+    hidden = torch.empty((n, F), dtype=torch.bfloat16, device=h.device)
+    _check(_fn("moe", "bn_moe_group")(h.data_ptr(), ld, ids.data_ptr(), wts.data_ptr(), work.data_ptr(), row_scale.data_ptr(),
+                                      xg.data_ptr(), T, D, E, K, MOE_TILE_ROWS, int(bool(weight_on_input)), _stream()),
+           "moe_group")
+    row_map, tiles = work.data_ptr() + 4 * n, work.data_ptr() + 8 * n
+    n_tiles = tiles + 12 * max_tiles
+    grouped = _fn("gemm_mfma", "bn_gemm_mfma_grouped")
+    _check(grouped(_code(torch.bfloat16), xg.data_ptr(), w_up.data_ptr(), hidden.data_ptr(), tiles, n_tiles, max_tiles, None, None,
+                   F * D, UNARY_ACTIVATIONS[activation], n, F, D, D, D, F, _stream()), "moe_experts_grouped(up)")
+    _check(grouped(_code(torch.float32), hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tiles, n_tiles, max_tiles, row_map,
+                   None if weight_on_input else row_scale.data_ptr(), D * F, -1, n, D, F, F, F, D, _stream()),
+           "moe_experts_grouped(down)")
     return PartialSums(y)
 
 

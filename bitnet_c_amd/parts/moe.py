@@ -8,9 +8,9 @@
       = sum over the chosen e of  w_e W_down,e act(W_up,e h)       weight_on "output"
 
 The experts' matrices are stacked on the device ([E, F, D] and [E, D, F]); the model folder holds them one by one
-(e<n>.w_up [F, D], e<n>.w_down [D, F]).  The router runs one wave a token and chooses on the device; steps of few rows
+(e<n>.w_up [F, D], e<n>.w_down [D, F]).  The router runs one workgroup a token and chooses on the device; steps of few rows
 read each chosen expert once per (token, choice) pair (ops.moe_experts), steps of many rows order the pairs by expert and
-run the two products on the matrix cores over tiles whose rows share an expert (ops.moe_experts_grouped).  Nothing waits
+run the two products as grouped matrix products over tiles whose rows share an expert (ops.moe_experts_grouped).  Nothing waits
 for the host, so the part's steps are captured like any other.  The result is handed on as the top_k slabs of float32
 rows (ops.PartialSums) that the consumer's kernel adds.
 """

@@ -304,10 +304,10 @@ def test_the_router_chooses_the_largest_scores(dtype, E, K, D):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("E,K,D,F,T", [(6, 2, 64, 32, 40), (3, 3, 48, 16, 9), (1, 1, 32, 8, 20), (9, 4, 96, 64, 70), (16, 1, 128, 64, 300)])
+@pytest.mark.parametrize("E,K,D,F,T", [(6, 2, 64, 32, 40), (3, 3, 48, 16, 9), (1, 1, 32, 8, 20), (9, 4, 96, 64, 70), (16, 1, 128, 64, 300), (4, 2, 72, 40, 700), (5, 1, 36, 20, 30)])
 def test_the_experts_compute_on_the_weighted_input(dtype, E, K, D, F, T):
-    """Every (token, choice) pair against expert(w h), summed over a token's choices; a pair a workgroup, and (bf16, sizes
-    in whole chunks of 32) the grouped products over pairs ordered by expert; the weight on the output as well."""
+    """Every (token, choice) pair against expert(w h), summed over a token's choices; a pair a workgroup, and (bf16, rows
+    of whole 16-byte groups) the grouped products over pairs ordered by expert; the weight on the output as well."""
     from bitnet_c_amd import ops
     g = torch.Generator().manual_seed(E + D + T)
     h = torch.randn(T, D, generator=g).to(dtype)
@@ -334,7 +334,7 @@ def test_the_experts_compute_on_the_weighted_input(dtype, E, K, D, F, T):
         if ops.moe_grouped_supported(T, D, F, dtype):
             y = ops.moe_experts_grouped(*args)
             close(y.slabs.sum(0), want, dtype)
-    assert ops.moe_grouped_supported(T, D, F, dtype) == (dtype == torch.bfloat16 and T >= 17 and D % 32 == 0 and F % 32 == 0)
+    assert ops.moe_grouped_supported(T, D, F, dtype) == (dtype == torch.bfloat16 and T >= 17 and D % 8 == 0 and F % 8 == 0)
 
 
 # ------------------------------------------------------------------------------------------------------------------

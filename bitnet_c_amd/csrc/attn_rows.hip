@@ -148,8 +148,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
         hi = pos0 + n_tok;                                        // exclusive
         lo = a.window > 0 ? max(0, pos0 + 1 - a.window) : 0;      // first key of the first row
         const int chunk = a.max_len ? bn_split_chunk(*a.max_len, a.n_splits) : a.chunk;
-        lo = max(lo, split * chunk);
-        hi = min(hi, (split + 1) * chunk);
+        // the splits of a windowed decode step are counted from the page of the window's first key: however long the
+        // sequence, its visible keys lie in the first window + BN_PAGE positions from there
+        const int base = (a.window > 0 && a.n_splits > 1 && !a.tiles) ? (lo / BN_PAGE) * BN_PAGE : 0;
+        lo = max(lo, base + split * chunk);
+        hi = min(hi, base + (split + 1) * chunk);
     }
 
     // phase C ownership: thread -> (jp, dp): keys jp, jp+JP, ...; output dims 2dp, 2dp+1

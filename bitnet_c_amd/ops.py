@@ -1199,6 +1199,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     n_splits > 1 the kernels then cut the keys into n_splits runs of split_chunk(max_len, n_splits) and
     `chunk` is not used, so that one captured launch serves every length up to the block table's width.
     v_transposed, blocked: the layout of the pages (neither: kernel_v_layout of qkv's type and hs).
+    window with n_splits > 1 (decode form on the vector kernel, bf16): the splits are counted from the page that holds the
+    window's first key, so n_splits * chunk need only cover window + PAGE positions, whatever the sequences' lengths.
     row_scale (decode form on the matrix cores with fused_rotate): a DeferredNorm whose factor the rows of qkv still
     lack (qkv is the product of its bf16 copy with the stacked weights); the kernel multiplies q and the new key and
     value of every row by it.
@@ -1268,7 +1270,10 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     if n_splits > 1:
         if chunk <= 0 or chunk % PAGE:
             raise KernelError(f"attention: chunk {chunk} must be a positive multiple of {PAGE}")
-        if n_splits * chunk < block_table.shape[1] * PAGE:
+        cover = block_table.shape[1] * PAGE
+        if window and decode and not use_mfma:           # the vector kernel counts a windowed step's splits from the window's first page
+            cover = min(cover, window + PAGE)
+        if n_splits * chunk < cover:
             raise KernelError(f"attention: {n_splits} splits of {chunk} keys do not cover the "
                               f"{block_table.shape[1]} pages of the block table")
         if n_splits > (1024 if fold else 64):

@@ -153,11 +153,18 @@ class Attention(Part):
         out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
         bias = (self.dist_a, self.dist_b) if self.distance_bias else None
         if ctx.is_decode:
-            n_splits, chunk = (1, 0) if self.window else ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype,
-                                                                           target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
+            if not self.window:
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
+            elif h.dtype == torch.bfloat16 and self.window >= 4 * ops.PAGE:
+                # a long window is cut like a sequence of its own length: the kernel counts the splits from the window's
+                # first page, so the plan depends on the window alone and serves every length (also a captured step's)
+                n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, self.window + ops.PAGE, h.dtype,
+                                                    target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
+            else:
+                n_splits, chunk = 1, 0                    # a short window is not split; a float32 cache sums in runs from position 0
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
-                          max_len_dev=ctx.max_len_dev if n_splits > 1 else None, v_transposed=True, blocked=False,
+                          max_len_dev=ctx.max_len_dev if n_splits > 1 and not self.window else None, v_transposed=True, blocked=False,
                           v_dim=vd, distance_bias=bias, sink=self.sink)
         elif (ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES and width % 8 == 0
               and qkv.data_ptr() % 16 == 0):

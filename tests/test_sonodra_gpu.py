@@ -192,8 +192,12 @@ def _run_window_case(dtype, H, G, hs, vd, T, window, qkv, scale, portions, matri
                           v_transposed=True)
         out = torch.full((n, H * vd), 9.0, dtype=dtype, device=DEV)
         if n == 1 and lo > 0:
-            ops.attention(rows, out, kp, vp, table, H, G, hs, scale, window=window, seq_lens=pos + 1, v_transposed=True,
-                          blocked=False, v_dim=vd)
+            n_splits, chunk = 1, 0
+            if window >= 4 * PAGE and dtype == torch.bfloat16:      # a long window is cut from its own first page on
+                n_splits, chunk = ops.decode_splits(1, H, G, window + PAGE, dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
+                assert n_splits > 1
+            ops.attention(rows, out, kp, vp, table, H, G, hs, scale, window=window, seq_lens=pos + 1, n_splits=n_splits,
+                          chunk=chunk, v_transposed=True, blocked=False, v_dim=vd)
         elif matrix_cores:
             qt = ops.GENERAL_PROMPT_TILE
             tiles = i32([[0, i, min(qt, n - i), lo + i] for i in range(0, n, qt)][::-1] + [[0, 0, 0, 0]])
@@ -209,12 +213,13 @@ def _run_window_case(dtype, H, G, hs, vd, T, window, qkv, scale, portions, matri
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window", [1, 2, 31, 64, 65, 100])
+@pytest.mark.parametrize("window", [1, 2, 31, 64, 65, 100, 300])
 def test_a_window_and_its_edges_on_the_vector_kernel(dtype, window):
     """Queries in prompt portions and decoded alone whose one outstanding key lies just inside the window (the oldest
-    visible position) or just outside it (one older): the first must carry the result, the second must not be seen."""
-    H, G, hs, vd, T, scale = 4, 2, 16, 24, 200, 0.3
-    queries = [3, 64, 70, 127, 128, 129, 140, 160, 180, 199]
+    visible position) or just outside it (one older): the first must carry the result, the second must not be seen.  The
+    long window's decode steps are cut into splits (bfloat16), which begin at the window's first page."""
+    H, G, hs, vd, T, scale = 4, 2, 16, 24, 200 if window < 256 else 720, 0.3
+    queries = [3, 64, 70, 127, 128, 129, 140, 160, 180, 199] + ([299, 300, 301, 383, 384, 450, 639, 640, 641, 719] if T > 200 else [])
     for inside in (True, False):
         spikes = [(i, i - window + (1 if inside else 0)) for i in queries]
         qkv, want = _window_case(dtype, H, G, hs, vd, T, window, 10 * window + inside, spikes, scale)
@@ -484,7 +489,7 @@ def test_long_decoding_with_peaked_attentions(tmp_path, dtype):
     carry the result), as a prompt in portions and then decoded for 80 tokens."""
     import bitnet_c_amd as bn
     cfg = dict(architecture="Sonodra", vocab=61, width=32, norm=dict(eps=1e-5), layers=[
-        _lat(2, 8, 8, 16, 1.5, _dense(48)), _att(2, 1, 8, 8, 1.5, 150, (10000.0, 4), None),
+        _lat(2, 8, 8, 16, 1.5, _dense(48)), _att(2, 1, 8, 8, 1.5, 300, (10000.0, 4), None),
         _lat(3, 4, 8, 16, 2.0, None, kv_from=0), _att(2, 2, 8, 4, 1.0, 64, None, _dense(40))])
     folder = write_folder(tmp_path / "peaked", cfg, 9)
     g = torch.Generator().manual_seed(2)
@@ -494,7 +499,7 @@ def test_long_decoding_with_peaked_attentions(tmp_path, dtype):
     want = ps.forward(ps.read_config(folder), ps.read_weights(folder), toks, angle_dtype=torch.float32)
     eng = engine(folder, dtype, max_tokens=4608)
     s, at, parts = eng.new_sequence(), 0, []
-    check = [0, 1, 63, 64, 65, 149, 150, 151, 2047, 2048, 2049, 2119]
+    check = [0, 1, 63, 64, 65, 299, 300, 301, 2047, 2048, 2049, 2119]
     for n in (1000, 1047, 73):
         w = [p - at for p in check if at <= p < at + n]
         parts.append(eng.step([bn.StepEntry(s, toks[at:at + n], w)]))

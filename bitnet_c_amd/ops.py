@@ -77,6 +77,9 @@ _SIGNATURES = {
         "bn_attn_general_supports": [c_int, c_int],
         "bn_attn_general_prompt": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                                    c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "bn_attn_general_decode": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
+                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                   c_void_p, c_void_p, c_void_p],
     },
     "state_mixers": {
         "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
@@ -1436,6 +1439,75 @@ def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torc
         block_table.data_ptr(), block_table.shape[1], tiles.data_ptr(), tiles.shape[0], H, Hkv, hs, v_dim, float(scale),
         da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), int(window),
         _stream()), "attention_general_prompt")
+
+
+def general_decode_plan(n_seqs: int, H: int, Hkv: int, max_len: int, window: int = 0):
+    """(n_splits, chunk, follows_length) for attention_general_decode: how a decode step's keys are cut so that the launch
+    fills the chip with its one-wave workgroups.  Without a window the plan follows max_len (the cache's bound in a
+    captured step: pass max_len_dev then, and the keys per split follow the longest sequence of each replay); with a window
+    it depends on the window alone, because the kernel counts the splits from the window's first page."""
+    if window:
+        n_splits, chunk = decode_splits(n_seqs, H, Hkv, window + PAGE, torch.bfloat16, target_wgs=VECTOR_DECODE_TARGET_WGS)
+        return n_splits, chunk, False
+    n_splits, chunk = decode_splits(n_seqs, H, Hkv, max_len, torch.bfloat16, target_wgs=VECTOR_DECODE_TARGET_WGS)
+    return n_splits, chunk, True
+
+
+def attention_general_decode(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                             block_table: torch.Tensor, seq_lens: torch.Tensor, H: int, Hkv: int, hs: int, v_dim: int, scale: float,
+                             *, window: int = 0, n_splits: int = 1, chunk: int = 0, max_len_dev=None, distance_bias=None,
+                             sink: bool = False) -> None:
+    """The decode form of attention_general_prompt (bf16, the same head sizes and pages): row b of qkv is sequence b's new
+    token, seq_lens [B] its keys in the cache (0: a padding row, whose output is zeros).  A wave takes the heads that share
+    a kv head together, so their keys and values are read once.  n_splits > 1 cuts the keys into runs of `chunk` positions
+    (a multiple of PAGE; with max_len_dev, a device int32, into runs of split_chunk(longest sequence, n_splits)), merged in
+    index order; with a window the runs are counted from the page of the window's first key and need only cover
+    window + PAGE positions.  distance_bias, sink: as attention()'s."""
+    require_gpu()
+    _dev(qkv, "qkv", torch.bfloat16, 2)
+    _dev(out, "out", torch.bfloat16, 2)
+    if not attention_general_supported(qkv.dtype, hs, v_dim):
+        raise KernelError(f"attention_general_decode: bf16 with head sizes from {_GENERAL_SIZES}, got {hs} and {v_dim}")
+    _check_pages(k_pages, v_pages, Hkv, hs, qkv.dtype, True, False, v_dim)
+    _dev(block_table, "block_table", torch.int32, 2)
+    _dev(seq_lens, "seq_lens", torch.int32, 1)
+    T = qkv.shape[0]
+    if (H % Hkv or qkv.shape[1] < H * hs or out.shape != (T, H * v_dim) or not out.is_contiguous() or seq_lens.numel() != T
+            or block_table.shape[0] < T or not block_table.is_contiguous() or not seq_lens.is_contiguous()):
+        raise KernelError(f"attention_general_decode: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} / seq_lens "
+                          f"{tuple(seq_lens.shape)} do not fit H={H} hs={hs} v_dim={v_dim}")
+    if window < 0 or _rows(qkv, "qkv") % 8 or qkv.data_ptr() % 16:
+        raise KernelError(f"attention_general_decode: window {window} / row stride {_rows(qkv, 'qkv')} (a multiple of 8, 16-byte aligned)")
+    da = db = None
+    if distance_bias is not None:
+        da, db = distance_bias
+        for t, nm in ((da, "distance_bias[0]"), (db, "distance_bias[1]")):
+            _dev(t, nm, torch.float32, 1)
+            if t.numel() != H or not t.is_contiguous():
+                raise KernelError(f"attention_general_decode: {nm} must hold one float32 per head")
+    part_o = part_ml = None
+    if n_splits > 1:
+        if max_len_dev is not None:
+            _dev(max_len_dev, "max_len_dev", torch.int32)
+            if max_len_dev.numel() != 1 or window:
+                raise KernelError("attention_general_decode: max_len_dev is one int32 and belongs to steps without a window")
+            chunk = split_chunk(block_table.shape[1] * PAGE, n_splits)
+        if chunk <= 0 or chunk % PAGE or n_splits > 64:
+            raise KernelError(f"attention_general_decode: chunk {chunk} must be a positive multiple of {PAGE}, at most 64 splits")
+        cover = min(block_table.shape[1] * PAGE, window + PAGE) if window else block_table.shape[1] * PAGE
+        if n_splits * chunk < cover:
+            raise KernelError(f"attention_general_decode: {n_splits} splits of {chunk} keys do not cover {cover} positions")
+        part_o = torch.empty((T * H * n_splits, v_dim), dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty((T * H * n_splits, 2), dtype=torch.float32, device=qkv.device)
+    if T == 0:
+        return
+    _check(_fn("attn_mfma_general", "bn_attn_general_decode")(
+        qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * v_dim, k_pages.data_ptr(), v_pages.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], seq_lens.data_ptr(), T, H, Hkv, hs, v_dim, float(scale),
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), int(window),
+        int(n_splits), int(chunk), part_o.data_ptr() if part_o is not None else None,
+        part_ml.data_ptr() if part_ml is not None else None,
+        max_len_dev.data_ptr() if (max_len_dev is not None and n_splits > 1) else None, _stream()), "attention_general_decode")
 
 
 # --------------------------------------------------------------------------------------

@@ -152,7 +152,15 @@ class Attention(Part):
                           v_transposed=True)
         out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
         bias = (self.dist_a, self.dist_b) if self.distance_bias else None
-        if ctx.is_decode:
+        on_matrix_cores = (ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES
+                           and width % 8 == 0 and qkv.data_ptr() % 16 == 0)
+        if ctx.is_decode and on_matrix_cores:
+            n_splits, chunk, follows = ops.general_decode_plan(ctx.n_rows, H, Hkv, kv.max_len, self.window)
+            ops.attention_general_decode(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, ctx.seq_lens, H, Hkv, hs, vd, self.scale,
+                                         window=self.window, n_splits=n_splits, chunk=chunk,
+                                         max_len_dev=ctx.max_len_dev if follows and n_splits > 1 else None,
+                                         distance_bias=bias, sink=self.sink)
+        elif ctx.is_decode:
             if not self.window:
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
             elif h.dtype == torch.bfloat16 and self.window >= 4 * ops.PAGE:
@@ -166,8 +174,7 @@ class Attention(Part):
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           max_len_dev=ctx.max_len_dev if n_splits > 1 and not self.window else None, v_transposed=True, blocked=False,
                           v_dim=vd, distance_bias=bias, sink=self.sink)
-        elif (ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES and width % 8 == 0
-              and qkv.data_ptr() % 16 == 0):
+        elif on_matrix_cores:
             ops.attention_general_prompt(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, vd, self.scale,
                                          ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self.sink,
                                          window=self.window)

@@ -92,12 +92,17 @@ class LatentAttention(Part):
                              ctx.seq_index, kv.block_table, kv.k_pages, kv.v_pages)
         q = ops.head_linear(p[:, :self.q_dim], self.uk)      # [T, H R]: the queries in the latent's space
         out = torch.empty((h.shape[0], H * R), dtype=h.dtype, device=h.device)
-        if ctx.is_decode:
+        on_matrix_cores = ops.attention_general_supported(h.dtype, R, R) and ops.GENERAL_PROMPT_ON_MATRIX_CORES
+        if ctx.is_decode and on_matrix_cores:
+            n_splits, chunk, _ = ops.general_decode_plan(ctx.n_rows, H, 1, kv.max_len)
+            ops.attention_general_decode(q, out, kv.k_pages, kv.v_pages, kv.block_table, ctx.seq_lens, H, 1, R, R, self.scale,
+                                         n_splits=n_splits, chunk=chunk, max_len_dev=ctx.max_len_dev if n_splits > 1 else None)
+        elif ctx.is_decode:
             n_splits, chunk = ops.decode_splits(ctx.n_rows, H, 1, kv.max_len, h.dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
             ops.attention(q, out, kv.k_pages, kv.v_pages, kv.block_table, H, 1, R, self.scale, seq_lens=ctx.seq_lens,
                           n_splits=n_splits, chunk=chunk, max_len_dev=ctx.max_len_dev if n_splits > 1 else None,
                           v_transposed=True, blocked=False, v_dim=R)
-        elif ops.attention_general_supported(h.dtype, R, R) and ops.GENERAL_PROMPT_ON_MATRIX_CORES:
+        elif on_matrix_cores:
             ops.attention_general_prompt(q, out, kv.k_pages, kv.v_pages, kv.block_table, H, 1, R, R, self.scale,
                                          ctx.tiles(ops.GENERAL_PROMPT_TILE))
         else:

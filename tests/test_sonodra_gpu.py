@@ -191,7 +191,11 @@ def _run_window_case(dtype, H, G, hs, vd, T, window, qkv, scale, portions, matri
         ops.qk_norm_store(rows, pos, H, G, hs, v_dim=vd, seq_index=i32([0] * n), block_table=table, k_pages=kp, v_pages=vp,
                           v_transposed=True)
         out = torch.full((n, H * vd), 9.0, dtype=dtype, device=DEV)
-        if n == 1 and lo > 0:
+        if n == 1 and lo > 0 and matrix_cores:
+            n_splits, chunk, _ = ops.general_decode_plan(1, H, G, table.shape[1] * PAGE, window)      # for what the table can hold
+            ops.attention_general_decode(rows, out, kp, vp, table, pos + 1, H, G, hs, vd, scale, window=window,
+                                         n_splits=n_splits, chunk=chunk)
+        elif n == 1 and lo > 0:
             n_splits, chunk = 1, 0
             if window >= 4 * PAGE and dtype == torch.bfloat16:      # a long window is cut from its own first page on
                 n_splits, chunk = ops.decode_splits(1, H, G, window + PAGE, dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
@@ -237,6 +241,56 @@ def test_a_window_and_its_edges_on_the_matrix_cores(H, G, hs, vd, window):
         qkv, want = _window_case(dtype, H, G, hs, vd, T, window, 7 * window + inside + hs, spikes, scale)
         got = _run_window_case(dtype, H, G, hs, vd, T, window, qkv, scale, (70, 80), True)
         close(got, want, dtype)
+
+
+@pytest.mark.parametrize("H,hs,T", [(16, 64, 330), (20, 256, 200), (5, 128, 700)])
+def test_many_heads_over_one_kv_head_on_the_matrix_cores(H, hs, T):
+    """No window, every head sharing the one kv head whose values are as wide as its keys (what a latent attention asks
+    for): prompt portions, then tokens one by one through the decode form with its keys in splits; single far keys carry
+    some of the queries."""
+    dtype, scale = torch.bfloat16, 1.0 / math.sqrt(hs)
+    spikes = [(i, j) for i, j in ((150, 0), (151, 63), (152, 64), (T - 1, 1), (T - 2, 65), (T - 3, 127), (T - 4, T - 5)) if j <= i]
+    qkv, want = _window_case(dtype, H, 1, hs, hs, T, 0, H + hs, spikes, scale)
+    got = _run_window_case(dtype, H, 1, hs, hs, T, 0, qkv, scale, (70, 80), True)
+    close(got, want, dtype)
+
+
+def test_decode_on_the_matrix_cores_a_batch_with_a_padding_row_and_the_length_on_the_device():
+    """Three rows of a decode step: a short sequence, a long one, a padding row (no keys: zeros); the keys per split
+    follow the longest sequence's length, which lies in device memory; a sink and a distance bias as well."""
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.cache import PAGE
+    dtype, H, G, hs, vd, scale = torch.bfloat16, 6, 2, 32, 64, 0.2
+    lens = [5, 300]
+    g = torch.Generator().manual_seed(3)
+    kp = torch.zeros(12, G, PAGE, hs, dtype=dtype, device=DEV)
+    vp = torch.zeros(12, G, vd, PAGE, dtype=dtype, device=DEV)
+    table = i32([[3, 0, 0, 0, 0, 0, 0, 0], [7, 1, 9, 4, 11, 0, 0, 0], [0, 0, 0, 0, 0, 0, 0, 0]])
+    da, db = 0.3 * torch.rand(H, generator=g), 0.1 + torch.rand(H, generator=g)
+    rows, wants = [], []
+    for b, n in enumerate(lens):
+        q, k, v = torch.randn(n, H, hs, generator=g), torch.randn(n, G, hs, generator=g), torch.randn(n, G, vd, generator=g)
+        qkv = torch.cat([q.reshape(n, -1), k.reshape(n, -1), v.reshape(n, -1)], 1).to(dtype)
+        ops.qk_norm_store(qkv.to(DEV), i32(list(range(n))), H, G, hs, v_dim=vd, seq_index=i32([b] * n), block_table=table,
+                          k_pages=kp, v_pages=vp, v_transposed=True)
+        qd = qkv[-1, :H * hs].double().view(H, hs)
+        kd, vd_ = qkv[:, H * hs:(H + G) * hs].double().view(n, G, hs), qkv[:, (H + G) * hs:].double().view(n, G, vd)
+        o = torch.zeros(H, vd, dtype=torch.float64)
+        for a in range(H):
+            sc = (kd[:, a // (H // G)] @ qd[a]) * scale - float(da[a]) * torch.log1p(float(db[a]) * torch.arange(n - 1, -1, -1, dtype=torch.float64))
+            e = torch.exp(sc - sc.max())
+            o[a] = (e @ vd_[:, a // (H // G)]) / (e.sum() + math.exp(-float(sc.max())))      # the sink: one more term of score 0
+        rows.append(qkv[-1])
+        wants.append(o.reshape(-1))
+    rows.append(torch.randn(H * hs + G * (hs + vd), generator=g).to(dtype))
+    q = torch.stack(rows).to(DEV)
+    for n_splits in (1, 4):
+        out = torch.full((3, H * vd), 5.0, dtype=dtype, device=DEV)
+        ops.attention_general_decode(q, out, kp, vp, table, i32(lens + [0]), H, G, hs, vd, scale, n_splits=n_splits,
+                                     chunk=2 * PAGE, max_len_dev=i32([300]) if n_splits > 1 else None,
+                                     distance_bias=(da.to(DEV), db.to(DEV)), sink=True)
+        close(out[:2], torch.stack(wants), dtype)
+        assert float(out[2].abs().max()) == 0.0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -54,6 +54,13 @@ CONFIGS = {
         _att(2, 1, 128, 128, 0.09, 100, (10000.0, 128), _moe(4, 1, 128)),
         _lat(2, 32, 64, 128, 0.15, _moe(16, 3, 32), kv_from=1),
         _lat(3, 32, 32, 128, 0.15, None, kv_from=1)]),
+    # sizes that fit no kernel's favourite shape: a width that is no multiple of 8, seven and 32 heads, a latent 96 wide,
+    # a rotation over 30 of 32 dimensions, a window of 33, three of eleven experts
+    "E": dict(architecture="Sonodra", vocab=90, width=100, norm=dict(eps=1e-6), layers=[
+        _lat(7, 18, 22, 96, 0.2, _moe(11, 3, 44)),
+        _att(14, 7, 32, 64, 0.17, 33, (1e6, 30), _dense(130)),
+        _att(8, 2, 96, 32, 0.1, 200, (1000.0, 96), _moe(5, 2, 72)),
+        _lat(32, 8, 8, 96, 0.3, None, kv_from=0)]),
     # ones everywhere: one head, a window of one token (a query sees itself alone), one expert, a latent as wide as a head
     "D": dict(architecture="Sonodra", vocab=40, width=32, norm=dict(eps=1e-5), layers=[
         _att(1, 1, 8, 8, 0.35, 1, (100.0, 8), _moe(1, 1, 8)),

@@ -118,6 +118,88 @@ __global__ __launch_bounds__(HL_COLS * HL_SLICES) void head_linear_kernel(HeadLi
     }
 }
 
+// The same product with 16-byte loads of the weights: a lane owns HLW_VEC consecutive output columns (8 bf16 or 4 float32),
+// O / HLW_VEC lanes cover a row of the head's matrix, and the 256 / (O / HLW_VEC) groups of lanes take the input dimension
+// in turn; their sums meet in shared memory.  One workgroup a (head, four rows of x): at one row a head's matrix is read
+// with sixteen loads a lane instead of one load an input row.
+#define HLW_ROWS 4
+#define HLW_THREADS 256
+
+template <typename T> struct HlwVec;
+template <> struct HlwVec<bf16> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void load(const bf16* p, float (&v)[8]) {
+        const uint4 w = *reinterpret_cast<const uint4*>(p);
+        v[0] = bf16lo_to_f32(w.x); v[1] = bf16hi_to_f32(w.x); v[2] = bf16lo_to_f32(w.y); v[3] = bf16hi_to_f32(w.y);
+        v[4] = bf16lo_to_f32(w.z); v[5] = bf16hi_to_f32(w.z); v[6] = bf16lo_to_f32(w.w); v[7] = bf16hi_to_f32(w.w);
+    }
+};
+template <> struct HlwVec<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const float4 w = *reinterpret_cast<const float4*>(p);
+        v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+    }
+};
+
+template <typename T>
+__global__ __launch_bounds__(HLW_THREADS) void head_linear_wide_kernel(HeadLinearArgs a) {
+    constexpr int V = HlwVec<T>::N;
+    extern __shared__ float xs[];                        // [HLW_ROWS][I], then the groups' sums [groups][HLW_ROWS][O]
+    float* red = xs + HLW_ROWS * a.I;
+    const int h = blockIdx.x, t0 = blockIdx.y * HLW_ROWS;
+    const int lanes = a.O / V, groups = HLW_THREADS / lanes;         // lanes <= 256
+    const int grp = threadIdx.x / lanes, cg = threadIdx.x - grp * lanes;
+    const int rows = min(HLW_ROWS, a.T - t0);
+    const T* x = reinterpret_cast<const T*>(a.x);
+    for (int idx = threadIdx.x; idx < HLW_ROWS * a.I; idx += HLW_THREADS) {
+        const int r = idx / a.I, i = idx - r * a.I;
+        xs[idx] = r < rows ? to_f32(x[(size_t)(t0 + r) * a.ldx + (size_t)h * a.I + i]) : 0.f;
+    }
+    __syncthreads();
+    float acc[HLW_ROWS][V];
+#pragma unroll
+    for (int r = 0; r < HLW_ROWS; ++r)
+#pragma unroll
+        for (int k = 0; k < V; ++k) acc[r][k] = 0.f;
+    if (grp < groups) {
+        const T* w = reinterpret_cast<const T*>(a.w) + (size_t)h * a.I * a.O + (size_t)cg * V;
+#pragma unroll 4
+        for (int i = grp; i < a.I; i += groups) {
+            float wv[V];
+            HlwVec<T>::load(w + (size_t)i * a.O, wv);
+#pragma unroll
+            for (int r = 0; r < HLW_ROWS; ++r) {
+                const float xv = xs[r * a.I + i];
+#pragma unroll
+                for (int k = 0; k < V; ++k) acc[r][k] = fmaf(xv, wv[k], acc[r][k]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < HLW_ROWS; ++r)
+#pragma unroll
+            for (int k = 0; k < V; ++k) red[((size_t)grp * HLW_ROWS + r) * a.O + cg * V + k] = acc[r][k];
+    }
+    __syncthreads();
+    T* y = reinterpret_cast<T*>(a.y);
+    const T* g = reinterpret_cast<const T*>(a.gate);
+    for (int idx = threadIdx.x; idx < rows * a.O; idx += HLW_THREADS) {
+        const int r = idx / a.O, o = idx - r * a.O;
+        float v = 0.f;
+        for (int k = 0; k < groups; ++k) v += red[((size_t)k * HLW_ROWS + r) * a.O + o];
+        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + (size_t)h * a.O + o])));
+        y[(size_t)(t0 + r) * a.ldy + (size_t)h * a.O + o] = from_f32<T>(v);
+    }
+}
+
+template <typename T>
+static bool hlw_takes(const void* w, int I, int O) {
+    constexpr int V = HlwVec<T>::N;
+    if (O % V || O / V > HLW_THREADS || ((uintptr_t)w & 15)) return false;
+    const int groups = HLW_THREADS / (O / V);
+    return (size_t)HLW_ROWS * ((size_t)I + (size_t)groups * O) * sizeof(float) <= 64 * 1024;
+}
+
 extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, void* y, int ldy, const void* gate, int ldg,
                               int n_rows, int H, int I, int O, hipStream_t s) {
     if (n_rows <= 0 || H <= 0 || I <= 0 || O <= 0 || !x || !w || !y) return BN_ERR_ARG;
@@ -126,6 +208,16 @@ extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, 
     if (row_tiles > 65535) return BN_ERR_ARG;
     HeadLinearArgs a;
     a.x = x; a.w = w; a.y = y; a.gate = gate; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.T = n_rows; a.H = H; a.I = I; a.O = O;
+    if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
+    const bool wide = dtype == BN_DT_F32 ? hlw_takes<float>(w, I, O) : hlw_takes<bf16>(w, I, O);
+    if (wide && (n_rows + HLW_ROWS - 1) / HLW_ROWS <= 65535) {
+        const int vec = dtype == BN_DT_F32 ? 4 : 8, groups = HLW_THREADS / (O / vec);
+        const dim3 wgrid(H, (n_rows + HLW_ROWS - 1) / HLW_ROWS);
+        const size_t wshm = (size_t)HLW_ROWS * ((size_t)I + (size_t)groups * O) * sizeof(float);
+        if (dtype == BN_DT_F32) hipLaunchKernelGGL(head_linear_wide_kernel<float>, wgrid, dim3(HLW_THREADS), wshm, s, a);
+        else hipLaunchKernelGGL(head_linear_wide_kernel<bf16>, wgrid, dim3(HLW_THREADS), wshm, s, a);
+        return bn_launch_status();
+    }
     const dim3 grid((O + HL_COLS - 1) / HL_COLS, H, row_tiles), block(HL_COLS * HL_SLICES);
     const size_t shm = (size_t)HL_ROWS * (I + HL_SLICES * HL_COLS) * sizeof(float);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(head_linear_kernel<float>, grid, block, shm, s, a);

@@ -148,6 +148,7 @@ template <>
 __device__ __forceinline__ float moe_row_dot<bf16>(const bf16* __restrict__ w, const float* __restrict__ x, int n, int lane) {
     float s = 0.f;
     if (n % 8 == 0 && ((uintptr_t)w & 15) == 0) {
+#pragma unroll 4
         for (int i = 8 * lane; i < n; i += 8 * BN_WAVE) {
             const uint4 p = *reinterpret_cast<const uint4*>(w + i);
             const float4 a = *reinterpret_cast<const float4*>(x + i), b = *reinterpret_cast<const float4*>(x + i + 4);
@@ -175,9 +176,18 @@ __global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_up_kernel(PairArgs 
     __syncthreads();
     const T* wu = reinterpret_cast<const T*>(a.w_up) + (size_t)e * a.F * a.D;
     const int f0 = blockIdx.x * MOE_PAIR_ROWS;
-    for (int f = f0 + wave; f < min(f0 + MOE_PAIR_ROWS, a.F); f += MOE_PAIR_THREADS / BN_WAVE) {
-        const float s = moe_row_dot<T>(wu + (size_t)f * a.D, xs, a.D, lane);
-        if (lane == 0) a.hidden[(size_t)pair * a.F + f] = to_f32(from_f32<T>(bn_unary_act(s, a.act)));
+    // a wave's two rows (MOE_PAIR_ROWS / 4) one after the other without a dependence between them: both rows' loads are
+    // in flight before the first sum is needed
+    float sums[MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE)];
+#pragma unroll
+    for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+        const int f = f0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+        sums[k] = f < a.F ? moe_row_dot<T>(wu + (size_t)f * a.D, xs, a.D, lane) : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+        const int f = f0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+        if (f < a.F && lane == 0) a.hidden[(size_t)pair * a.F + f] = to_f32(from_f32<T>(bn_unary_act(sums[k], a.act)));
     }
 }
 
@@ -194,9 +204,16 @@ __global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_down_kernel(PairArg
     const T* wd = reinterpret_cast<const T*>(a.w_down) + (size_t)e * a.D * a.F;
     float* y = a.y + ((size_t)j * a.T + t) * a.D;
     const int d0 = blockIdx.x * MOE_PAIR_ROWS;
-    for (int d = d0 + wave; d < min(d0 + MOE_PAIR_ROWS, a.D); d += MOE_PAIR_THREADS / BN_WAVE) {
-        const float s = moe_row_dot<T>(wd + (size_t)d * a.F, hid, a.F, lane);
-        if (lane == 0) y[d] = s * out_scale;
+    float sums[MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE)];
+#pragma unroll
+    for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+        const int d = d0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+        sums[k] = d < a.D ? moe_row_dot<T>(wd + (size_t)d * a.F, hid, a.F, lane) : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+        const int d = d0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+        if (d < a.D && lane == 0) y[d] = sums[k] * out_scale;
     }
 }
 
